@@ -30,9 +30,12 @@ def register_architecture(name: str, config_from_dict, build_spec) -> None:
 
 def architecture_name(config: Mapping[str, Any], where: str = "config.json") -> str:
     archs = config.get("architectures") or []
-    if not archs:
-        raise ConfigError(f"no 'architectures' field in {where}")
-    return archs[0]
+    if archs:
+        return archs[0]
+    one = config.get("architecture")        # some configurations name their one architecture as a string
+    if isinstance(one, str) and one:
+        return one
+    raise ConfigError(f"no 'architectures' field in {where}")
 
 
 def get_architecture(name: str) -> Architecture:

@@ -1,4 +1,4 @@
-// Paged causal attention, generic path: any head size up to 512, any head counts,
+// Paged causal attention, generic path: any head size up to 640, any head counts,
 // any page size, float or bf16 storage, all arithmetic in float.  It is the kernel
 // of the 32-bit path and the fallback of the bf16 path for shapes the MFMA kernel
 // refuses.  One 64-lane block per (token, q head); keys are walked in tiles of 64
@@ -11,7 +11,7 @@
 // Cache layout: K pages[page][kv_head][slot][D], V pages[page][kv_head][D][slot].
 #include "common.h"
 
-#define GEN_MAX_E 8  // head size up to 64 * 8
+#define GEN_MAX_E 10  // head size up to 64 * 10
 
 template <typename T>
 __global__ void __launch_bounds__(64)

@@ -1,0 +1,304 @@
+// Routed experts: choice of experts per token, rows grouped by expert on the device, and the two
+// grouped matrix products of gated experts.  Nothing here returns to the host: a step's routing is
+// known only on the device, so every launch is sized by upper bounds and blocks without work leave.
+//
+//   route:   z = router logits (float) -> the `top` largest per token (lowest index among equals),
+//            weight = sigmoid(z)
+//   group:   entry s = token * top + kk  ->  position in a list ordered by expert; tiles of MOE_TM rows
+//            that never straddle two experts
+//   gate/up: z[pos] = act(w g) * (w u),  g = Wg[e] x[token], u = Wu[e] x[token]      (w = the entry's weight
+//            when it scales the expert's INPUT: w (W x) = W (w x); else 1)
+//   down:    y[kk][token] = (Wd[e] z[pos]) * (w if it scales the OUTPUT else 1)        float
+// The order of rows inside an expert's group depends on timing; no result does: every output row is a
+// sum over the inner size in ascending order, alone.
+#include "common.h"
+
+#define MOE_TM 64
+#define MOE_TN 64
+#define MOE_BK 16
+
+// one thread per token
+__global__ void moe_route_kernel(const float* __restrict__ logits, int n, int experts, int top,
+                                 int* __restrict__ ids, float* __restrict__ weights) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const float* z = logits + (long long)t * experts;
+  for (int kk = 0; kk < top; ++kk) {
+    int best = -1;
+    float bz = -INFINITY;
+    for (int e = 0; e < experts; ++e) {
+      const float v = z[e];
+      if (!(v > bz) && best >= 0) continue;
+      bool taken = false;
+      for (int p = 0; p < kk; ++p) taken |= ids[(long long)t * top + p] == e;
+      if (!taken) { best = e; bz = v; }
+    }
+    if (best < 0) best = 0;        // rows of NaN: some expert, the NaN shows in the output
+    ids[(long long)t * top + kk] = best;
+    weights[(long long)t * top + kk] = 1.f / (1.f + expf(-z[best]));
+  }
+}
+
+// Router and choice in one launch: one block per token, the token's row in LDS as floats, a wave per
+// expert (in turns) sums its products lane by lane and then across the wave: float logits whatever the
+// activation type, the same order of additions whatever the batch.  logits_out (may be null) [n, experts].
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, int hidden, int experts, int top,
+                  int* __restrict__ ids, float* __restrict__ weights, float* __restrict__ logits_out) {
+  extern __shared__ float rs[];      // x [hidden] | z [experts]
+  float* xs = rs;
+  float* z = rs + hidden;
+  const long long t = blockIdx.x;
+  const int lane = threadIdx.x & (JV_WAVE - 1), wid = threadIdx.x / JV_WAVE, nw = blockDim.x / JV_WAVE;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) xs[c] = to_f32(x[t * hidden + c]);
+  __syncthreads();
+  for (int e = wid; e < experts; e += nw) {
+    const T* w = W + (long long)e * hidden;
+    float acc = 0.f;
+    for (int c = lane; c < hidden; c += JV_WAVE) acc = fmaf(xs[c], to_f32(w[c]), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      z[e] = acc;
+      if (logits_out) logits_out[t * experts + e] = acc;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int kk = 0; kk < top; ++kk) {
+      int best = -1;
+      float bz = -INFINITY;
+      for (int e = 0; e < experts; ++e) {
+        const float v = z[e];
+        if (!(v > bz) && best >= 0) continue;
+        bool taken = false;
+        for (int p = 0; p < kk; ++p) taken |= ids[t * top + p] == e;
+        if (!taken) { best = e; bz = v; }
+      }
+      if (best < 0) best = 0;
+      ids[t * top + kk] = best;
+      weights[t * top + kk] = 1.f / (1.f + expf(-z[best]));
+    }
+  }
+}
+
+// One block.  meta: [0] number of tiles; offsets [experts + 1]; tile_expert / tile_row0 [max_tiles];
+// order [entries]: entry index at each position; rank [entries] scratch.
+__global__ void __launch_bounds__(1024)
+moe_group_kernel(const int* __restrict__ ids, int entries, int experts, int* __restrict__ meta,
+                 int* __restrict__ offsets, int* __restrict__ tile_expert, int* __restrict__ tile_row0,
+                 int* __restrict__ order, int* __restrict__ rank) {
+  extern __shared__ int sh[];      // count [experts] | start [experts + 1] | first tile [experts + 1]
+  int* count = sh;
+  int* start = sh + experts;
+  int* tile0 = start + experts + 1;
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int s = threadIdx.x; s < entries; s += blockDim.x) rank[s] = atomicAdd(&count[ids[s]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tiles = 0;
+    for (int e = 0; e < experts; ++e) {
+      start[e] = at;
+      tile0[e] = tiles;
+      at += count[e];
+      tiles += (count[e] + MOE_TM - 1) / MOE_TM;
+    }
+    start[experts] = at;
+    tile0[experts] = tiles;
+    meta[0] = tiles;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e <= experts; e += blockDim.x) offsets[e] = start[e];
+  for (int e = threadIdx.x; e < experts; e += blockDim.x)
+    for (int i = tile0[e]; i < tile0[e + 1]; ++i) {
+      tile_expert[i] = e;
+      tile_row0[i] = start[e] + (i - tile0[e]) * MOE_TM;
+    }
+  for (int s = threadIdx.x; s < entries; s += blockDim.x) order[start[ids[s]] + rank[s]] = s;
+}
+
+// grid (max tiles, column tiles of the expert width).  x [tokens, hidden]; Wg, Wu [experts, ff, hidden];
+// z [entries, ff] by position.
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_gate_up_kernel(T* __restrict__ z, const T* __restrict__ x, const T* __restrict__ Wg, const T* __restrict__ Wu,
+                   const int* __restrict__ meta, const int* __restrict__ offsets, const int* __restrict__ tile_expert,
+                   const int* __restrict__ tile_row0, const int* __restrict__ order, const float* __restrict__ weights,
+                   int top, int hidden, int ff, int act, int scale_input) {
+  if ((int)blockIdx.x >= meta[0]) return;
+  __shared__ float As[MOE_BK][MOE_TM + 4];
+  __shared__ float Gs[MOE_BK][MOE_TN + 4];
+  __shared__ float Us[MOE_BK][MOE_TN + 4];
+  __shared__ int tok[MOE_TM];
+  __shared__ float wgt[MOE_TM];
+  const int e = tile_expert[blockIdx.x], row0 = tile_row0[blockIdx.x];
+  const int rows = min(MOE_TM, offsets[e + 1] - row0);
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int n0 = blockIdx.y * MOE_TN;
+  if (tid < MOE_TM) {
+    const int s = tid < rows ? order[row0 + tid] : -1;
+    tok[tid] = s < 0 ? -1 : s / top;
+    wgt[tid] = (s < 0 || !scale_input) ? 1.f : weights[s];
+  }
+  __syncthreads();
+  const T* G = Wg + (long long)e * ff * hidden;
+  const T* U = Wu + (long long)e * ff * hidden;
+  float ag[4][4] = {}, au[4][4] = {};
+  for (int k0 = 0; k0 < hidden; k0 += MOE_BK) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int idx = tid + q * 256;
+      const int r = idx >> 4, kk = idx & 15, k = k0 + kk;
+      const int tk = tok[r], wn = n0 + r;
+      As[kk][r] = (tk >= 0 && k < hidden) ? to_f32(x[(long long)tk * hidden + k]) : 0.f;
+      const bool in = wn < ff && k < hidden;
+      Gs[kk][r] = in ? to_f32(G[(long long)wn * hidden + k]) : 0.f;
+      Us[kk][r] = in ? to_f32(U[(long long)wn * hidden + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < MOE_BK; ++kk) {
+      float a[4], g[4], u[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { g[j] = Gs[kk][tx * 4 + j]; u[j] = Us[kk][tx * 4 + j]; }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          ag[i][j] = fmaf(a[i], g[j], ag[i][j]);
+          au[i][j] = fmaf(a[i], u[j], au[i][j]);
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = ty * 4 + i;
+    if (m >= rows) continue;
+    const float w = wgt[m];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < ff) z[(long long)(row0 + m) * ff + n] = from_f32<T>(jv_gated(act, ag[i][j] * w, au[i][j] * w));
+    }
+  }
+}
+
+// grid (max tiles, column tiles of hidden).  z [entries, ff] by position; Wd [experts, hidden, ff];
+// y [top, tokens, hidden] float.
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_down_kernel(float* __restrict__ y, const T* __restrict__ z, const T* __restrict__ Wd, const int* __restrict__ meta,
+                const int* __restrict__ offsets, const int* __restrict__ tile_expert, const int* __restrict__ tile_row0,
+                const int* __restrict__ order, const float* __restrict__ weights, int top, int n_tokens, int hidden,
+                int ff, int scale_output) {
+  if ((int)blockIdx.x >= meta[0]) return;
+  __shared__ float As[MOE_BK][MOE_TM + 4];
+  __shared__ float Ws[MOE_BK][MOE_TN + 4];
+  __shared__ int ent[MOE_TM];
+  const int e = tile_expert[blockIdx.x], row0 = tile_row0[blockIdx.x];
+  const int rows = min(MOE_TM, offsets[e + 1] - row0);
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int n0 = blockIdx.y * MOE_TN;
+  if (tid < MOE_TM) ent[tid] = tid < rows ? order[row0 + tid] : -1;
+  __syncthreads();
+  const T* W = Wd + (long long)e * hidden * ff;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < ff; k0 += MOE_BK) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int idx = tid + q * 256;
+      const int r = idx >> 4, kk = idx & 15, k = k0 + kk;
+      const int wn = n0 + r;
+      As[kk][r] = (r < rows && k < ff) ? to_f32(z[(long long)(row0 + r) * ff + k]) : 0.f;
+      Ws[kk][r] = (wn < hidden && k < ff) ? to_f32(W[(long long)wn * ff + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < MOE_BK; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = ty * 4 + i;
+    if (m >= rows) continue;
+    const int s = ent[m];
+    const int token = s / top, kk = s - token * top;
+    const float w = scale_output ? weights[s] : 1.f;
+    float* o = y + ((long long)kk * n_tokens + token) * hidden;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < hidden) o[n] = acc[i][j] * w;
+    }
+  }
+}
+
+extern "C" int jv_moe_tile_rows() { return MOE_TM; }
+
+extern "C" int jv_moe_route(const float* logits, int n, int experts, int top, int* ids, float* weights, void* stream) {
+  if (n <= 0) return 0;
+  if (experts <= 0 || top <= 0 || top > experts) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((n + 127) / 128), dim3(128), 0, (hipStream_t)stream, logits, n, experts,
+                     top, ids, weights);
+  return JV_LAUNCH_CHECK();
+}
+
+extern "C" int jv_moe_group(const int* ids, int entries, int experts, int* meta, int* offsets, int* tile_expert,
+                            int* tile_row0, int* order, int* rank, void* stream) {
+  if (entries <= 0) return 0;
+  if (experts <= 0 || experts > 4096) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (3 * experts + 2) * sizeof(int), (hipStream_t)stream, ids,
+                     entries, experts, meta, offsets, tile_expert, tile_row0, order, rank);
+  return JV_LAUNCH_CHECK();
+}
+
+#define DEFINE_MOE(SUF, T)                                                                                        \
+  extern "C" int jv_moe_router_##SUF(const void* x, const void* W, int n, int hidden, int experts, int top,       \
+                                     int* ids, float* weights, float* logits_out, void* stream) {                 \
+    if (n <= 0) return 0;                                                                                         \
+    if (experts <= 0 || top <= 0 || top > experts || hidden <= 0 || (hidden + experts) > 15000)                   \
+      return (int)hipErrorInvalidValue;                                                                           \
+    hipLaunchKernelGGL(moe_router_kernel<T>, dim3(n), dim3(256), (hidden + experts) * sizeof(float),              \
+                       (hipStream_t)stream, (const T*)x, (const T*)W, hidden, experts, top, ids, weights,         \
+                       logits_out);                                                                               \
+    return JV_LAUNCH_CHECK();                                                                                     \
+  }                                                                                                               \
+  extern "C" int jv_moe_gate_up_##SUF(void* z, const void* x, const void* Wg, const void* Wu, const int* meta,    \
+                                      const int* offsets, const int* tile_expert, const int* tile_row0,           \
+                                      const int* order, const float* weights, int max_tiles, int top, int hidden, \
+                                      int ff, int act, int scale_input, void* stream) {                           \
+    if (max_tiles <= 0 || ff <= 0) return 0;                                                                      \
+    if (!jv_act_known(act) || (ff + MOE_TN - 1) / MOE_TN > 65535) return (int)hipErrorInvalidValue;               \
+    hipLaunchKernelGGL(moe_gate_up_kernel<T>, dim3(max_tiles, (ff + MOE_TN - 1) / MOE_TN), dim3(256), 0,          \
+                       (hipStream_t)stream, (T*)z, (const T*)x, (const T*)Wg, (const T*)Wu, meta, offsets,        \
+                       tile_expert, tile_row0, order, weights, top, hidden, ff, act, scale_input);                \
+    return JV_LAUNCH_CHECK();                                                                                     \
+  }                                                                                                               \
+  extern "C" int jv_moe_down_##SUF(float* y, const void* z, const void* Wd, const int* meta, const int* offsets,  \
+                                   const int* tile_expert, const int* tile_row0, const int* order,                \
+                                   const float* weights, int max_tiles, int top, int n_tokens, int hidden,        \
+                                   int ff, int scale_output, void* stream) {                                      \
+    if (max_tiles <= 0 || hidden <= 0) return 0;                                                                  \
+    if ((hidden + MOE_TN - 1) / MOE_TN > 65535) return (int)hipErrorInvalidValue;                                 \
+    hipLaunchKernelGGL(moe_down_kernel<T>, dim3(max_tiles, (hidden + MOE_TN - 1) / MOE_TN), dim3(256), 0,         \
+                       (hipStream_t)stream, y, (const T*)z, (const T*)Wd, meta, offsets, tile_expert, tile_row0,  \
+                       order, weights, top, n_tokens, hidden, ff, scale_output);                                  \
+    return JV_LAUNCH_CHECK();                                                                                     \
+  }
+
+DEFINE_MOE(bf16, bf16_t)
+DEFINE_MOE(f32, float)

@@ -37,7 +37,7 @@ def parse_args(argv=None):
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens live requests hold at any time (per request rounded up to the page size)")
     p.add_argument("--block-size", type=int, default=16, help="tokens per cache page (default 16)")
-    p.add_argument("--max-num-seqs", type=int, default=8, help="state slots / live requests (default 8)")
+    p.add_argument("--max-num-seqs", type=int, default=4, help="state slots / live requests (default 4)")
     return p.parse_args(argv)
 
 

@@ -312,7 +312,7 @@ def paged_attention_generic(out, q, q_row_stride, k_pages, v_pages, block_tables
     _need(out.shape == (n, nq * head_dim) and out.dtype == q.dtype, "out must be [tokens, nq * D] of q's type")
     _need(q.numel() >= (n - 1) * q_row_stride + nq * head_dim if n else True, "q is too small for its stride")
     _need(nkv > 0 and nq % nkv == 0, "q heads must be a multiple of kv heads")
-    _need(head_dim <= 512, "head size above 512 is not supported")
+    _need(head_dim <= 640, "head size above 640 is not supported")
     page_size = k_pages.shape[2]
     _check_pages(k_pages, v_pages, q.dtype, nkv, page_size, head_dim)
     _need(block_tables.dim() == 2, "block_tables must be [requests, pages]")
@@ -785,3 +785,261 @@ def calibrate_mfma(sink: torch.Tensor, turns: int, blocks: int) -> float:
     lib.jv_calibrate_mfma_flops.restype = ctypes.c_double
     _check(lib.jv_calibrate_mfma(_ptr(sink), c_int(turns), c_int(blocks), _stream()), "calibrate_mfma")
     return float(lib.jv_calibrate_mfma_flops(c_int(blocks), c_int(turns)))
+
+
+# --------------------------------------------------------------------------- norms around a sublayer's output
+class PendingNorm:
+    """A sublayer's output ``y`` (rows of the activation type, or None) plus float partial results
+    ``parts`` [P, rows, hidden] (or None) whose sum still has to be normed with ``weight`` before it
+    joins the residual stream: what a layer arrangement that norms the output of its sublayers hands
+    to the next norm, which does both in one pass (``postnorm_add_rmsnorm``)."""
+
+    def __init__(self, y, parts, weight: torch.Tensor, eps: float):
+        self.y, self.parts, self.weight, self.eps = y, parts, weight, float(eps)
+
+
+def split_sublayer_output(out):
+    """(rows or None, float stack or None) of what a mixer or feed-forward returned: rows of the
+    activation type, a float stack of partial results, or already a pair of both."""
+    if isinstance(out, tuple):
+        return out
+    if out.dim() == 3:
+        return None, out
+    return out, None
+
+
+def postnorm_add_rmsnorm(h, y, parts, post_weight, eps: float, weight=None, out=None, rows=None,
+                         out_eps: float | None = None) -> None:
+    """h += norm(y + parts[0] + parts[1] + ...; post_weight) in the float residual stream, then, with
+    ``out``, out = norm(h; weight) (with ``out_eps``, default ``eps``) in the activation type.  With ``rows`` (int32 indices) only those
+    rows are computed and h is left alone.  y is [rows of h, hidden] in the activation type or None,
+    parts a float32 stack [P, rows of h, hidden] or None (any P)."""
+    _dev(h, y, parts, post_weight, weight, out, rows)
+    _f32(h, "h")
+    n, hidden = h.shape
+    _f32(post_weight, "post_weight", hidden)
+    _need(y is not None or parts is not None, "nothing to add")
+    _need(hidden <= 16384, "rows wider than 16,384 are not supported")
+    if y is not None:
+        _need(y.shape == h.shape, "y must match h's shape")
+    if parts is not None:
+        _need(parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[1:] == h.shape,
+              "parts must be float32 [P, *h.shape]")
+    if out is not None:
+        _f32(weight, "weight", hidden)
+        n_out = out.shape[0]
+        _need(out.shape[-1] == hidden, "out width differs from h")
+        _need(y is None or y.dtype == out.dtype, "y and out must have one type")
+    else:
+        _need(rows is None, "rows without an output change nothing")
+        n_out = n
+    if rows is None:
+        _need(n_out == n, "out must have one row per row of h")
+    else:
+        _i32(rows, "rows", n_out)
+    kind = out.dtype if out is not None else (y.dtype if y is not None else torch.float32)
+    fn = getattr(library.core(), f"jv_postnorm_add_rmsnorm_{_suffix(kind)}")
+    _check(fn(_ptr(h), _ptr(y), _ptr(parts), c_int(0 if parts is None else parts.shape[0]),
+              c_longlong(0 if parts is None else parts.stride(0)), _ptr(post_weight), _ptr(weight), _ptr(out),
+              _ptr(rows), c_int(n_out), c_int(hidden), c_float(eps), c_float(eps if out_eps is None else out_eps), _stream()),
+           "postnorm_add_rmsnorm")
+
+
+def gated_rmsnorm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """norm(o; weight) * sigmoid(gate) for float rows ``o`` [n, width]; ``gate`` is a [n, width] view (unit
+    column stride, any row stride) of the activation type, which is also the result's."""
+    _dev(o, weight)
+    _f32(o, "o")
+    n, width = o.shape
+    _f32(weight, "weight", width)
+    _need(gate.is_cuda and gate.shape == o.shape and gate.stride(1) == 1, "gate must be a [n, width] view with unit column stride")
+    out = torch.empty((n, width), dtype=gate.dtype, device=o.device)
+    fn = getattr(library.core(), f"jv_gated_rmsnorm_{_suffix(gate.dtype)}")
+    _check(fn(_ptr(out), _ptr(o), _ptr(gate), c_longlong(gate.stride(0)), _ptr(weight), c_int(n), c_int(width),
+              c_float(eps), _stream()), "gated_rmsnorm")
+    return out
+
+
+# --------------------------------------------------------------------------- attention over a cached latent
+def rope_table_amp(positions: torch.Tensor, inv_freq: torch.Tensor, amplitude: float) -> torch.Tensor:
+    """``rope_table`` with cos and sin multiplied by a constant."""
+    _dev(positions, inv_freq)
+    n, half = positions.numel(), inv_freq.numel()
+    _i32(positions, "positions")
+    _f32(inv_freq, "inv_freq")
+    out = torch.empty((n, 2 * half), dtype=torch.float32, device=positions.device)
+    _check(library.core().jv_rope_table_amp(_ptr(out), _ptr(positions), _ptr(inv_freq), c_int(n), c_int(half),
+                                            c_float(amplitude), _stream()), "rope_table_amp")
+    return out
+
+
+def latent_prepare(proj, q_rank: int, rank: int, rot: int, rot_dims: int, q_weight, kv_weight, eps: float, cos_sin,
+                   slot_mapping, k_pages, v_pages, page_size: int) -> torch.Tensor:
+    """From rows ``proj`` = [q latent | kv latent | key part to rotate | ...]: returns the normed q latent
+    [n, q_rank]; stores [normed kv latent | rotated key part] of every token with a slot (>= 0) into its key
+    page [pages, 1, page_size, rank + rot] and transposed value page [pages, 1, rank + rot, page_size]."""
+    _dev(proj, q_weight, kv_weight, cos_sin, slot_mapping, k_pages, v_pages)
+    n, ld = proj.shape
+    _need(ld >= q_rank + rank + rot, "proj rows are too short")
+    _f32(q_weight, "q_weight", q_rank)
+    _f32(kv_weight, "kv_weight", rank)
+    _need(rot_dims % 2 == 0 and 0 <= rot_dims <= rot, "the rotated size must be even and at most the key part")
+    if rot_dims:
+        _f32(cos_sin, "cos_sin", n * rot_dims)
+    if k_pages is not None:
+        _i32(slot_mapping, "slot_mapping", n)
+        _check_pages(k_pages, v_pages, proj.dtype, 1, page_size, rank + rot)
+    cq = torch.empty((n, q_rank), dtype=proj.dtype, device=proj.device)
+    fn = getattr(library.core(), f"jv_latent_prepare_{_suffix(proj.dtype)}")
+    _check(fn(_ptr(proj), c_longlong(ld), c_int(n), c_int(q_rank), c_int(rank), c_int(rot), c_int(rot_dims),
+              _ptr(q_weight), _ptr(kv_weight), c_float(eps), _ptr(cos_sin),
+              _ptr(slot_mapping if k_pages is not None else None), _ptr(cq), _ptr(k_pages), _ptr(v_pages),
+              c_int(page_size), _stream()), "latent_prepare")
+    return cq
+
+
+def latent_query_rope(q, qe, heads: int, dim: int, rot: int, rot_dims: int, rank: int, cos_sin) -> None:
+    """qe[t, h, rank:] = rotate(q[t, h, dim:]) for q [n, heads * (dim + rot)], qe [n, heads * (rank + rot)]."""
+    _dev(q, qe, cos_sin)
+    n = q.shape[0]
+    _need(q.shape == (n, heads * (dim + rot)) and qe.shape == (n, heads * (rank + rot)) and q.dtype == qe.dtype,
+          "q must be [n, heads * (dim + rot)], qe [n, heads * (rank + rot)] of one type")
+    if rot_dims:
+        _f32(cos_sin, "cos_sin", n * rot_dims)
+    fn = getattr(library.core(), f"jv_latent_query_rope_{_suffix(q.dtype)}")
+    _check(fn(_ptr(q), _ptr(qe), c_int(n), c_int(heads), c_int(dim), c_int(rot), c_int(rot_dims), c_int(rank),
+              _ptr(cos_sin), _stream()), "latent_query_rope")
+
+
+def head_linear(y, y_head_stride: int, x, x_head_stride: int, w, gate=None) -> None:
+    """One matrix per head: y[t, h * ys : h * ys + N] = w[h] @ x[t, h * xs : h * xs + K], w [heads, N, K];
+    with ``gate`` (a [n, heads * N] view with unit column stride) the result is multiplied by sigmoid(gate).
+    x and y are row-major matrices of the activation type; float accumulation."""
+    _dev(y, x, w)
+    heads, N, K = w.shape
+    n = x.shape[0]
+    _need(x.dtype == w.dtype == y.dtype, "x, w and y must have one type")
+    _need(y.shape[0] == n, "x and y differ in rows")
+    _need((heads - 1) * x_head_stride + K <= x.shape[1] and (heads - 1) * y_head_stride + N <= y.shape[1],
+          "heads do not fit the rows")
+    if gate is not None:
+        _need(gate.is_cuda and gate.dtype == x.dtype and gate.shape == (n, heads * N) and gate.stride(1) == 1,
+              "gate must be a [n, heads * N] view with unit column stride")
+    fn = getattr(library.core(), f"jv_head_linear_{_suffix(x.dtype)}")
+    _check(fn(_ptr(y), c_longlong(y.shape[1]), c_int(y_head_stride), _ptr(x), c_longlong(x.shape[1]),
+              c_int(x_head_stride), _ptr(w), c_int(n), c_int(N), c_int(K), c_int(heads), _ptr(gate),
+              c_longlong(0 if gate is None else gate.stride(0)), _stream()), "head_linear")
+
+
+# --------------------------------------------------------------------------- linear attention with decay
+LIGHTNING_CHUNK_MIN_TOKENS = 8     # from this many tokens of a request on, the kernel by chunks
+
+
+def lightning_max_dim(chunks: bool) -> int:
+    return library.core().jv_lightning_max_dim(c_int(1 if chunks else 0))
+
+
+def lightning_attention(proj, q_off: int, k_off: int, v_off: int, state, slot_ids, cu_seqlens, decay, heads: int,
+                        dim: int, vdim: int, chunks: bool) -> torch.Tensor:
+    """Float [n, heads * vdim]: o_t = S_t^T q_t with S_t = decay_h S_(t-1) + k_t v_t^T per request and head,
+    q, k, v = silu of the columns of ``proj`` at the given offsets (head by head).  ``state``
+    [slots + 1, heads, dim, vdim] float holds S of every request before the step and after it.
+    ``chunks``: the kernel that takes a request's tokens 32 at a time instead of one by one."""
+    _dev(proj, state, slot_ids, cu_seqlens, decay)
+    n, ld = proj.shape
+    r = slot_ids.numel()
+    _i32(slot_ids, "slot_ids")
+    _i32(cu_seqlens, "cu_seqlens", r + 1)
+    _f32(decay, "decay", heads)
+    _f32(state, "state")
+    _need(state.dim() == 4 and tuple(state.shape[1:]) == (heads, dim, vdim), "state must be [slots, heads, dim, vdim]")
+    _need(max(q_off, k_off) + heads * dim <= ld and v_off + heads * vdim <= ld, "proj rows are too short")
+    _need(dim <= lightning_max_dim(chunks), f"key size {dim} above the kernel's {lightning_max_dim(chunks)}")
+    out = torch.empty((n, heads * vdim), dtype=torch.float32, device=proj.device)
+    fn = getattr(library.core(), f"jv_lightning_{_suffix(proj.dtype)}")
+    _check(fn(_ptr(out), _ptr(proj), c_longlong(ld), c_int(q_off), c_int(k_off), c_int(v_off), _ptr(state),
+              _ptr(slot_ids), _ptr(cu_seqlens), _ptr(decay), c_int(r), c_int(heads), c_int(dim), c_int(vdim),
+              c_int(1 if chunks else 0), _stream()), "lightning_attention")
+    return out
+
+
+# --------------------------------------------------------------------------- routed experts
+def moe_tile_rows() -> int:
+    return library.core().jv_moe_tile_rows()
+
+
+class MoePlan:
+    """Device-side grouping of a step's (token, choice) entries by expert."""
+
+    def __init__(self, ids, weights, meta, offsets, tile_expert, tile_row0, order, max_tiles, top):
+        self.ids, self.weights, self.meta, self.offsets = ids, weights, meta, offsets
+        self.tile_expert, self.tile_row0, self.order, self.max_tiles, self.top = tile_expert, tile_row0, order, max_tiles, top
+
+
+def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, logits_out=None) -> MoePlan:
+    """Chooses for every token the ``top`` experts with the largest router logits (weights sigmoid(logit);
+    the lowest index among equal logits) and orders the n * top entries by expert, all on the device.
+    Either float ``logits`` [n, experts] are given, or rows ``x`` [n, hidden] and the router matrix
+    ``w_router`` [experts, hidden] of one type: then the logits are made in the same launch, in float
+    (``logits_out``, float32 [n, experts], receives them if given)."""
+    if logits is not None:
+        _dev(logits)
+        _f32(logits, "logits")
+        n, experts = logits.shape
+        dev = logits.device
+    else:
+        _dev(x, w_router, logits_out)
+        n, hidden = x.shape
+        experts = w_router.shape[0]
+        _need(w_router.shape == (experts, hidden) and w_router.dtype == x.dtype, "the router must be [experts, hidden] of x's type")
+        _need(hidden + experts <= 15000, "row and router too wide for the router kernel")
+        if logits_out is not None:
+            _f32(logits_out, "logits_out", n * experts)
+        dev = x.device
+    _need(0 < top <= experts, "top must be between 1 and the number of experts")
+    entries = n * top
+    max_tiles = -(-entries // moe_tile_rows()) + experts
+    ints = torch.empty(entries * 3 + 1 + experts + 1 + 2 * max_tiles, dtype=torch.int32, device=dev)
+    ids, rank, order = ints[:entries], ints[entries:2 * entries], ints[2 * entries:3 * entries]
+    at = 3 * entries
+    meta, offsets = ints[at:at + 1], ints[at + 1:at + 2 + experts]
+    at += 2 + experts
+    tile_expert, tile_row0 = ints[at:at + max_tiles], ints[at + max_tiles:at + 2 * max_tiles]
+    weights = torch.empty(entries, dtype=torch.float32, device=dev)
+    lib = library.core()
+    if logits is not None:
+        _check(lib.jv_moe_route(_ptr(logits), c_int(n), c_int(experts), c_int(top), _ptr(ids), _ptr(weights), _stream()),
+               "moe_route")
+    else:
+        _check(getattr(lib, f"jv_moe_router_{_suffix(x.dtype)}")(
+            _ptr(x), _ptr(w_router), c_int(n), c_int(hidden), c_int(experts), c_int(top), _ptr(ids), _ptr(weights),
+            _ptr(logits_out), _stream()), "moe_router")
+    _check(lib.jv_moe_group(_ptr(ids), c_int(entries), c_int(experts), _ptr(meta), _ptr(offsets), _ptr(tile_expert),
+                            _ptr(tile_row0), _ptr(order), _ptr(rank), _stream()), "moe_group")
+    return MoePlan(ids, weights, meta, offsets, tile_expert, tile_row0, order, max_tiles, top)
+
+
+def moe_experts(x, plan: MoePlan, w_gate, w_up, w_down, activation: str, out: torch.Tensor,
+                weight_on_input: bool = True) -> None:
+    """out[kk, t] = down[e] (act(gate[e] xs) * (up[e] xs)) for the kk-th chosen expert e of token t, float32
+    [top, n, hidden]; xs = weight * x[t] with ``weight_on_input``, else x[t] and the result is multiplied
+    by the weight.  w_gate, w_up [experts, ff, hidden], w_down [experts, hidden, ff]."""
+    _dev(x, w_gate, w_up, w_down, out)
+    n, hidden = x.shape
+    experts, ff, _ = w_gate.shape
+    _need(w_gate.shape == w_up.shape == (experts, ff, hidden) and w_down.shape == (experts, hidden, ff),
+          "expert weights must be [experts, ff, hidden] and [experts, hidden, ff]")
+    _need(x.dtype == w_gate.dtype == w_up.dtype == w_down.dtype, "x and the weights must have one type")
+    _need(out.dtype == torch.float32 and tuple(out.shape) == (plan.top, n, hidden), "out must be float32 [top, n, hidden]")
+    _need(plan.ids.numel() == n * plan.top, "the plan belongs to another step")
+    z = torch.empty((n * plan.top, ff), dtype=x.dtype, device=x.device)
+    lib, suf = library.core(), _suffix(x.dtype)
+    p = plan
+    _check(getattr(lib, f"jv_moe_gate_up_{suf}")(
+        _ptr(z), _ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(p.meta), _ptr(p.offsets), _ptr(p.tile_expert),
+        _ptr(p.tile_row0), _ptr(p.order), _ptr(p.weights), c_int(p.max_tiles), c_int(p.top), c_int(hidden), c_int(ff),
+        c_int(_gate_act_id(activation)), c_int(1 if weight_on_input else 0), _stream()), "moe_gate_up")
+    _check(getattr(lib, f"jv_moe_down_{suf}")(
+        _ptr(out), _ptr(z), _ptr(w_down), _ptr(p.meta), _ptr(p.offsets), _ptr(p.tile_expert), _ptr(p.tile_row0),
+        _ptr(p.order), _ptr(p.weights), c_int(p.max_tiles), c_int(p.top), c_int(n), c_int(hidden), c_int(ff),
+        c_int(0 if weight_on_input else 1), _stream()), "moe_down")

@@ -144,7 +144,8 @@ def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, window: int, device) -> Mfm
 
 
 def run(att, out, qkv, ctx, mem) -> None:
-    q_row_stride = (att.nq + 2 * att.nkv) * att.d
+    # q heads of a row sit at the front of the fused q/k/v projection, unless the mixer says where else
+    q_row_stride = getattr(att, "q_row_stride", None) or (att.nq + 2 * att.nkv) * att.d
     if not K.mfma_attention_supported(qkv.dtype, att.d, ctx.page_size):
         K.paged_attention_generic(
             out, qkv, q_row_stride, mem.pages["k"], mem.pages["v"], ctx.block_tables[mem.group], ctx.token_req,

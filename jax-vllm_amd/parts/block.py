@@ -54,4 +54,49 @@ def _add_norm(norm, h, delta, reader, n_rows: int):
     return norm.add_norm(h, delta)
 
 
+class SandwichBlock:
+    """Every sublayer between two norms:
+
+        h = h + norm_1b(mixer(norm_1(h)));   h = h + norm_2b(feed_forward(norm_2(h)))
+
+    (the second line only for a layer that has a feed-forward).  A sublayer's output is handed on as a
+    ``K.PendingNorm`` (the output and the norm weight that belongs to it): the next norm's kernel norms it,
+    adds it to the stream and norms the stream in one pass, also across the border of two layers and
+    before the head."""
+
+    def __init__(self, norm: PartSpec, has_feed_forward: bool = True,
+                 names=("norm1", "norm1b", "norm2", "norm2b")):
+        self.has_feed_forward = bool(has_feed_forward)
+        self.names = tuple(names) if self.has_feed_forward else tuple(names[:2])
+        self.norms = [build_part("norm", norm) for _ in self.names]
+
+    @property
+    def replayable(self) -> bool:
+        return all(is_replayable(n) for n in self.norms)
+
+    def tensors(self) -> dict:
+        out = {}
+        for name, part in zip(self.names, self.norms):
+            for k, v in part.tensors().items():
+                out[f"{name}.{k}"] = v
+        return out
+
+    def bind(self, tensors: dict, dtype: torch.dtype) -> None:
+        for name, part in zip(self.names, self.norms):
+            part.bind({k[len(name) + 1:]: v for k, v in tensors.items() if k.startswith(name + ".")}, dtype)
+
+    def forward(self, h, delta, mixer, feed_forward, ctx, mem):
+        from ..ops import kernels as K
+
+        x = self.norms[0].add_norm(h, delta)
+        a = mixer.forward(x, ctx, mem)
+        pending = K.PendingNorm(*K.split_sublayer_output(a), self.norms[1].weight, self.norms[1].eps)
+        if not self.has_feed_forward:
+            return pending
+        y = self.norms[2].add_norm(h, pending)
+        f = feed_forward.forward(y, ctx)
+        return K.PendingNorm(*K.split_sublayer_output(f), self.norms[3].weight, self.norms[3].eps)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "sandwich", SandwichBlock)

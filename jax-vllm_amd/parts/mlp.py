@@ -21,6 +21,7 @@ class GatedMLP:
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.activation = activation
         self.w_gate_up = self.w_down = None
+        self.partial_out = True     # whether the result may be a float stack of partial products (the next norm adds them)
 
     def tensors(self) -> dict:
         h, i = self.hidden_size, self.intermediate_size
@@ -41,7 +42,7 @@ class GatedMLP:
 
     def forward(self, x, ctx=None) -> torch.Tensor:
         z = K.linear(x, self.w_gate_up, gate_pairs=self.activation)    # gate and up rows alternate in the fused weight
-        return K.linear(z, self.w_down, partial_ok=True)   # the next norm adds the partial products
+        return K.linear(z, self.w_down, partial_ok=self.partial_out)   # the next norm adds the partial products
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

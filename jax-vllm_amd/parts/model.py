@@ -23,12 +23,14 @@ class Layer:
     def __init__(self, spec: LayerSpec):
         self.spec = spec
         self.mixer = build_part("mixer", spec.mixer)
-        self.feed_forward = build_part("feed_forward", spec.feed_forward)
+        self.feed_forward = build_part("feed_forward", spec.feed_forward) if spec.feed_forward is not None else None
         self.block = build_part("block", spec.block)
-        self._members = (
-            (spec.mixer_prefix, self.mixer),
-            (spec.feed_forward_prefix, self.feed_forward),
-            ("", self.block),
+        self._members = tuple(
+            (sub, part) for sub, part in (
+                (spec.mixer_prefix, self.mixer),
+                (spec.feed_forward_prefix, self.feed_forward),
+                ("", self.block),
+            ) if part is not None
         )
 
     def _name(self, sub: str, local: str) -> str:
@@ -72,33 +74,36 @@ class DecoderModel:
     def tensor_specs(self) -> dict:
         """Checkpoint name -> TensorSpec of every tensor the model loads."""
         s = self.spec
-        out = {s.embedding_prefix + k: v for k, v in self.embedding.tensors().items()}
+        out = {self._name(s.embedding_prefix + k): v for k, v in self.embedding.tensors().items()}
         for layer in self.layers:
             out.update(layer.tensors())
-        out.update({s.final_norm_prefix + k: v for k, v in self.final_norm.tensors().items()})
+        out.update({self._name(s.final_norm_prefix + k): v for k, v in self.final_norm.tensors().items()})
         if not s.tie_head_to_embedding:
-            out.update({s.head_prefix + k: v for k, v in self.head.tensors().items()})
+            out.update({self._name(s.head_prefix + k): v for k, v in self.head.tensors().items()})
         return out
+
+    def _name(self, name: str) -> str:
+        return self.spec.rename.get(name, name)
 
     def ignored_tensor_names(self) -> set:
         """Names a checkpoint may hold that are deliberately not read (a tied head's own copy)."""
         s = self.spec
-        return {s.head_prefix + k for k in self.head.tensors()} if s.tie_head_to_embedding else set()
+        return {self._name(s.head_prefix + k) for k in self.head.tensors()} if s.tie_head_to_embedding else set()
 
     def bind(self, tensors: dict, dtype: torch.dtype) -> None:
         """Hand every part its tensors (already on the device, already in their final types)."""
         s = self.spec
         self.dtype = dtype
-        emb = {k: tensors[s.embedding_prefix + k] for k in self.embedding.tensors()}
+        emb = {k: tensors[self._name(s.embedding_prefix + k)] for k in self.embedding.tensors()}
         self.embedding.bind(emb, dtype)
         self.device = next(iter(emb.values())).device
         for layer in self.layers:
             layer.bind(tensors, dtype)
-        self.final_norm.bind({k: tensors[s.final_norm_prefix + k] for k in self.final_norm.tensors()}, dtype)
+        self.final_norm.bind({k: tensors[self._name(s.final_norm_prefix + k)] for k in self.final_norm.tensors()}, dtype)
         if s.tie_head_to_embedding:
             self.head.bind(emb, dtype)  # the same buffer, no copy
         else:
-            self.head.bind({k: tensors[s.head_prefix + k] for k in self.head.tensors()}, dtype)
+            self.head.bind({k: tensors[self._name(s.head_prefix + k)] for k in self.head.tensors()}, dtype)
 
     # ---- memory
     def memory_plan(self) -> list:
@@ -114,7 +119,7 @@ class DecoderModel:
         parts = [self.embedding, self.final_norm, self.head]
         for run in self.spec.schedule:
             layer = self.layers[run.layer]
-            parts += [layer.mixer, layer.feed_forward, layer.block]
+            parts += [p for p in (layer.mixer, layer.feed_forward, layer.block) if p is not None]
         return all(is_replayable(p) for p in parts)
 
     # ---- one step

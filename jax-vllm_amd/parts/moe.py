@@ -1,0 +1,73 @@
+"""Routed experts: a feed-forward of many small gated feed-forwards, of which each token uses a few
+(no reference counterpart).
+
+    z = W_router x  (float);   s = sigmoid(z);   the ``top`` experts with the largest scores are chosen
+    out = sum over the chosen e of  expert_e(s_e * x)   [+ shared(x)]
+    expert(u) = W_down ( act(W_gate u) * (W_up u) )
+
+The score multiplies the expert's INPUT (``weight_on_input``; with False it multiplies the output).  Since
+the products are linear, s (W u) is computed instead of W (s u): in float, after the product.  Routing,
+the grouping of rows by expert and the two grouped products all run on the device (``ops.kernels.moe_*``).
+The result is handed on as (rows of the shared expert or None, float stack [top, tokens, hidden] of the
+chosen experts' outputs); the next norm adds them in that order.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..ops import kernels as K
+from .spec import PartSpec, TensorSpec, build_part, is_replayable, register_part
+
+
+class RoutedExperts:
+    def __init__(self, hidden_size: int, num_experts: int, top: int, expert_size: int, activation: str = "silu",
+                 weight_on_input: bool = True, shared: Optional[PartSpec] = None,
+                 expert_names=("gate", "up", "down")):
+        if activation not in K.GATE_ACTIVATIONS:
+            raise ValueError(f"the expert kernels have {sorted(K.GATE_ACTIVATIONS)}, not {activation!r}")
+        self.hidden_size, self.experts, self.top, self.ff = int(hidden_size), int(num_experts), int(top), int(expert_size)
+        if not 0 < self.top <= self.experts:
+            raise ValueError(f"top = {self.top} of {self.experts} experts")
+        self.activation, self.weight_on_input = activation, bool(weight_on_input)
+        self.names = tuple(expert_names)
+        self.shared = build_part("feed_forward", shared) if shared is not None else None
+        if self.shared is not None and hasattr(self.shared, "partial_out"):
+            self.shared.partial_out = False     # its rows are added beside the experts' float stack
+
+    @property
+    def replayable(self) -> bool:
+        return self.shared is None or is_replayable(self.shared)
+
+    def tensors(self) -> dict:
+        g, u, d = self.names
+        t = {"router.weight": TensorSpec((self.experts, self.hidden_size))}
+        for e in range(self.experts):
+            t[f"experts.{e}.{g}.weight"] = TensorSpec((self.ff, self.hidden_size))
+            t[f"experts.{e}.{u}.weight"] = TensorSpec((self.ff, self.hidden_size))
+            t[f"experts.{e}.{d}.weight"] = TensorSpec((self.hidden_size, self.ff))
+        if self.shared is not None:
+            for k, v in self.shared.tensors().items():
+                t["shared." + k] = v
+        return t
+
+    def bind(self, tensors: dict, dtype: torch.dtype) -> None:
+        g, u, d = self.names
+        self.w_router = tensors["router.weight"]
+        self.w_gate = torch.stack([tensors[f"experts.{e}.{g}.weight"] for e in range(self.experts)]).contiguous()
+        self.w_up = torch.stack([tensors[f"experts.{e}.{u}.weight"] for e in range(self.experts)]).contiguous()
+        self.w_down = torch.stack([tensors[f"experts.{e}.{d}.weight"] for e in range(self.experts)]).contiguous()
+        if self.shared is not None:
+            self.shared.bind({k[len("shared."):]: v for k, v in tensors.items() if k.startswith("shared.")}, dtype)
+
+    def forward(self, x, ctx=None):
+        n = x.shape[0]
+        plan = K.moe_route(None, self.top, x=x, w_router=self.w_router)
+        out = torch.empty((self.top, n, self.hidden_size), dtype=torch.float32, device=x.device)
+        K.moe_experts(x, plan, self.w_gate, self.w_up, self.w_down, self.activation, out, self.weight_on_input)
+        rows = self.shared.forward(x, ctx) if self.shared is not None else None
+        return rows, out
+
+
+register_part("feed_forward", "routed_experts", RoutedExperts)

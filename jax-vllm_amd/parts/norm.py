@@ -34,12 +34,19 @@ class RMSNorm:
 
     def add_norm(self, h: torch.Tensor, delta, rows=None, unscaled_ok: bool = False):
         """The residual step fused with the norm: ``h += delta`` in the float residual stream,
-        returns ``norm(h)`` in the activation type.  With ``rows`` only those rows are normed
+        returns ``norm(h)`` in the activation type.  ``delta`` may be a ``K.PendingNorm``: then what is
+        added is its own norm of the sublayer's output.  With ``rows`` only those rows are normed
         and ``h`` is left alone.  With ``unscaled_ok`` the reader multiplies the rows by a matrix
         through ``K.linear`` and nothing else: for the few rows of a decode step whose ``delta``
         comes as partial products the result may then be ``K.UnscaledRows`` (``h * weight`` with
         the scale left to that product's epilogue), whose residual step is shared out to many blocks
         a row."""
+        if isinstance(delta, K.PendingNorm):
+            # a sublayer's output that is normed on its own before it joins the stream: both norms in one pass
+            n_out = h.shape[0] if rows is None else rows.numel()
+            out = torch.empty((n_out, self.size), dtype=self.dtype, device=h.device)
+            K.postnorm_add_rmsnorm(h, delta.y, delta.parts, delta.weight, delta.eps, self.weight, out, rows, out_eps=self.eps)
+            return out
         if (unscaled_ok and rows is None and delta is not None and delta.dim() == 3
                 and K.unscaled_rows_possible(self.dtype, h.shape[0], self.size)):
             return K.add_parts_unscaled(h, delta, self.weight, self.eps)

@@ -10,6 +10,8 @@ attention-input kernel, which takes that table and this part's flags.
 """
 from __future__ import annotations
 
+import math
+
 import torch
 
 from ..ops import kernels as K
@@ -19,13 +21,17 @@ from .spec import register_part
 class RotaryEncoding:
     replayable = True      # the table is computed on the device from the step's positions
 
-    def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None, interleaved: bool = False):
+    def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None, interleaved: bool = False,
+                 rescale: dict | None = None):
         self.head_dim = int(head_dim)
         self.theta = float(theta)
         self.rotary_dim = int(rotary_dim) if rotary_dim is not None else self.head_dim
         self.interleaved = bool(interleaved)
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and at most the head size {self.head_dim}")
+        # frequencies rescaled for contexts longer than the ``original`` one (YaRN): see ``inverse_frequencies``
+        self.rescale = dict(rescale) if rescale else None
+        self.amplitude = 0.1 * math.log(float(self.rescale["factor"])) + 1.0 if self.rescale else 1.0
         self.inv_freq = None
 
     def tensors(self) -> dict:
@@ -34,7 +40,23 @@ class RotaryEncoding:
     def inverse_frequencies(self) -> torch.Tensor:
         """float32 table of rotary_dim/2 entries, computed as the reference does."""
         d = self.rotary_dim
-        return 1.0 / (self.theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        if self.rescale is None:
+            return 1.0 / (self.theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+        # With ``rescale`` = {factor, original, fast, slow}: a pair that makes more than ``fast`` turns over
+        # the original context keeps its frequency, one that makes fewer than ``slow`` turns is slowed down
+        # by ``factor``, and the pairs between are blended linearly by their index; cos and sin are then
+        # scaled by ``amplitude`` = 0.1 ln(factor) + 1.  Computed in double, rounded once.
+        r = self.rescale
+        i = torch.arange(d // 2, dtype=torch.float64)
+        f = self.theta ** (-2.0 * i / d)
+
+        def pair_with_turns(t: float) -> float:
+            return d * math.log(float(r["original"]) / (2 * math.pi * t)) / (2 * math.log(self.theta))
+
+        lo = max(math.floor(pair_with_turns(float(r["fast"]))), 0)
+        hi = min(math.ceil(pair_with_turns(float(r["slow"]))), d - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0, 1)
+        return (f / float(r["factor"]) * ramp + f * (1 - ramp)).to(torch.float32)
 
     def bind(self, tensors: dict, dtype: torch.dtype, device=None) -> None:
         self.inv_freq = self.inverse_frequencies().to(device or "cuda").contiguous()
@@ -47,10 +69,14 @@ class RotaryEncoding:
 
     def rotation_table(self, ctx):
         """Float cos/sin table of the step's positions for the attention-input kernel."""
-        key = ("rope_table", self.theta, self.rotary_dim)
+        key = ("rope_table", self.theta, self.rotary_dim, tuple(sorted(self.rescale.items())) if self.rescale else None)
         table = ctx.extras.get(key)
         if table is None:
-            table = ctx.extras[key] = K.rope_table(ctx.positions, self.inv_freq)
+            if self.rescale is None:
+                table = K.rope_table(ctx.positions, self.inv_freq)
+            else:
+                table = K.rope_table_amp(ctx.positions, self.inv_freq, self.amplitude)
+            ctx.extras[key] = table
         return table
 
 

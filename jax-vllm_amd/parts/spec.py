@@ -210,7 +210,7 @@ class LayerSpec:
 
     prefix: str                    # e.g. "model.layers.3."
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: Optional[PartSpec]   # None: a layer without a feed-forward (its block must be built for that)
     block: PartSpec
     mixer_prefix: str = ""         # below ``prefix``, e.g. "self_attn."
     feed_forward_prefix: str = ""  # below ``prefix``, e.g. "mlp."
@@ -242,6 +242,9 @@ class ModelSpec:
     layers: Sequence[LayerSpec]
     schedule: Sequence[LayerRun]
     tie_head_to_embedding: bool = False
+    # checkpoint name of a tensor outside the layers (embedding, final norm, head) where it differs from
+    # prefix + the part's local name
+    rename: Mapping[str, str] = field(default_factory=dict)
 
     def __post_init__(self):
         for i, run in enumerate(self.schedule):
