@@ -37,6 +37,32 @@ SHAPES = {
     "32b": ("Qwen3-32B-shaped", dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64,
                                      intermediate_size=25600)),
 }
+
+
+def lomozen_shape(width, layers, heads, experts, top, expert_ff, shared_ff, vocab=32000, window=1024):
+    """A Lomozen configuration with layer sizes of a real model's order: of every four layers one is lightning
+    attention and three are latent attention (a cached vector of 224 + 32 elements), every layer has routed experts."""
+    latent = {"type": "latent_attention", "mixer": {
+        "heads": heads, "dim": 64, "rot_dim": 32, "vdim": 64, "kv_rank": 224, "q_rank": width // 4 + 256,
+        "scale": 96 ** -0.5, "mask": {"size": window},
+        "rot": {"base": 500000.0, "dims": 32, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    lightning = {"type": "lightning", "mixer": {"heads": heads, "dim": 128, "vdim": 128,
+                                                "decay": [1.0 - 2.0 ** (-5 - 3 * h / heads) for h in range(heads)]}}
+    mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff}, "shared": {"ff": shared_ff}}
+    return {"architecture": "Lomozen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "layers": [dict(lightning if i % 4 == 0 else latent, mlp=mlp) for i in range(layers)]}
+
+
+# --only design: Lomozen beside the dense model of the same width, depth, vocabulary and feed-forward
+# parameters per token (top * expert + shared = intermediate)
+DESIGN_SHAPES = {
+    "2k": (lomozen_shape(2048, 8, 16, 32, 4, 512, 1024),
+           dict(QWEN3_8B, num_hidden_layers=8, hidden_size=2048, num_attention_heads=16, num_key_value_heads=4,
+                head_dim=128, intermediate_size=3072, vocab_size=32000)),
+    "4k": (lomozen_shape(4096, 8, 32, 64, 6, 1024, 2048),
+           dict(QWEN3_8B, num_hidden_layers=8, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                head_dim=128, intermediate_size=8192, vocab_size=32000)),
+}
 PROMPT_LEN = 1024
 MAX_CONTEXT = 8192
 PREFILL_TOKENS = 2048
@@ -133,6 +159,65 @@ def kernel_shares(run) -> dict:
         totals[group] = totals.get(group, 0.0) + t
     whole = sum(totals.values()) or 1.0
     return {g: round(t / whole, 4) for g, t in sorted(totals.items(), key=lambda kv: -kv[1])}
+
+
+def kernel_times(run, top: int = 14) -> dict:
+    """Microseconds of GPU time by kernel name while ``run()`` executes, the ``top`` largest and the total."""
+    from torch.profiler import ProfilerActivity, profile
+
+    sync()
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        run()
+        sync()
+    rows = {}
+    for e in prof.key_averages():
+        t = float(getattr(e, "self_device_time_total", 0.0))
+        if t > 0.0 and not str(e.device_type).endswith("CPU"):
+            name = e.key.split("(")[0].split("<")[0].replace("void ", "")[:48]
+            rows[name] = rows.get(name, 0.0) + t
+    out = {k: round(v, 1) for k, v in sorted(rows.items(), key=lambda kv: -kv[1])[:top]}
+    out["total"] = round(sum(rows.values()), 1)
+    return out
+
+
+def measure_design(args, rng):
+    """Lomozen and the dense model of equal size through the same engine: prefill of 2,048 tokens, decode at
+    batch 8 and 32 from 1,024-token prompts, and where the GPU's time goes in one prefill and in decode steps."""
+    from jax_vllm_amd import LLM, SamplingParams
+    from jax_vllm_amd.engine.entries import StepEntry
+
+    out = {"shape": args.design_shape, "dtype": args.dtype, "prefill_tokens": PREFILL_TOKENS, "decode_prompt_len": PROMPT_LEN}
+    for name, cfg in zip(("lomozen", "dense"), DESIGN_SHAPES[args.design_shape]):
+        vocab = cfg.get("vocab") or cfg["vocab_size"]
+        llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=16, max_num_seqs=32, max_model_len=4096,
+                  num_blocks=1 + 32 * (2048 // 16) + 256, max_num_batched_tokens=PREFILL_TOKENS, enable_prefix_cache=False)
+        res = {"layers": len(llm.model.layers)}
+        pre_s = measure_prefill(llm, rng, vocab)
+        res["prefill_tokens_per_s"] = round(PREFILL_TOKENS / pre_s, 1)
+        res["prefill_ms"] = round(pre_s * 1e3, 3)
+        for b in (8, 32):
+            tps, step_s, _ = measure_decode(llm, b, args.steps if args.steps <= 128 else 128, min(args.warmup, 8), rng, vocab)
+            res[f"decode_b{b}_tokens_per_s"] = round(tps, 1)
+            res[f"decode_b{b}_ms_per_step"] = round(step_s * 1e3, 4)
+        if not args.no_kernel_share:
+            toks = rng.integers(0, vocab, size=PREFILL_TOKENS).tolist()
+            llm.core.start_request("share")
+            res["prefill_kernels_us"] = kernel_times(lambda: llm.core.run([StepEntry("share", toks, [PREFILL_TOKENS - 1])]))
+            llm.core.finish_request("share")
+            for _ in range(8):
+                llm.add_request(rng.integers(0, vocab, size=PROMPT_LEN).tolist(), SamplingParams(max_new_tokens=64))
+            while any(r.num_remaining > 1 or not r.output_ids for r in llm.scheduler.running) or llm.scheduler.waiting:
+                llm.step()
+            for _ in range(4):
+                llm.step()
+            res["decode_b8_kernels_us_8_steps"] = kernel_times(lambda: [llm.step() for _ in range(8)])
+            llm.abort_all()
+        out[name] = res
+        del llm
+        import torch
+
+        torch.cuda.empty_cache()
+    return out
 
 
 def calibrate(device="cuda") -> dict:
@@ -265,12 +350,16 @@ def main():
     ap.add_argument("--tune-library", action="store_true",
                     help="prewarm the engine with the matrix library timing its own kernels (steps of more than 64 rows)")
     ap.add_argument("--no-kernel-share", action="store_true", help="leave out the per-kernel time shares")
-    ap.add_argument("--only", choices=["prefill", "decode", "mixed", "long-prompt", "ttft", "calibrate"], default=None,
+    ap.add_argument("--design-shape", choices=sorted(DESIGN_SHAPES), default="2k",
+                    help="with --only design: the width of both models (2,048 or 4,096), 8 layers each")
+    ap.add_argument("--only", choices=["prefill", "decode", "mixed", "long-prompt", "ttft", "calibrate", "design"], default=None,
                     help="run one phase alone and print its result (for profiling); mixed: 32 running decodes "
                          "joined by 4 prompts of 3,000 tokens in portions of 512 under a budget of 2,048; "
                          "long-prompt: one prompt of --prompt-len tokens (default 32,768) in portions of 2,048; "
                          "ttft: time to first token of a 2,048-token prompt, cold and with its first 1,024 tokens "
-                         "in the cache; calibrate: the plain read and matrix-core rates of this box")
+                         "in the cache; calibrate: the plain read and matrix-core rates of this box; design: the Lomozen "
+                         "architecture (latent and lightning attention, routed experts) beside the dense model of "
+                         "equal size: prefill, decode and the kernels' times of both")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--prompt-len", type=int, default=None,
                     help="with --only decode: prompt length of the decoding requests (long-context runs, default "
@@ -298,6 +387,9 @@ def main():
     block = 16
     if args.only == "calibrate":
         print(json.dumps(calibrate()), flush=True)
+        return
+    if args.only == "design":
+        print(json.dumps(measure_design(args, rng)), flush=True)
         return
     if args.only == "ttft":
         llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=block, max_num_seqs=4, max_model_len=4096,

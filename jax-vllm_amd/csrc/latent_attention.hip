@@ -156,6 +156,56 @@ head_linear_kernel(T* __restrict__ y, long long ldy, int ys, const T* __restrict
   }
 }
 
+// The same for at most HL_ROWS rows (decode steps): a block takes 64 outputs of one head against all rows, the
+// rows of x in LDS as floats; thread (n, part) sums its quarter of the inner size for every row, the quarters
+// are added in their order.  Every W element is read once.
+#define HL_ROWS 16
+template <typename T>
+__global__ void __launch_bounds__(256)
+head_linear_rows_kernel(T* __restrict__ y, long long ldy, int ys, const T* __restrict__ x, long long ldx, int xs,
+                        const T* __restrict__ W, int M, int N, int K, const T* __restrict__ g, long long ldg) {
+  extern __shared__ float hl[];          // x [M][K] | partial sums [4][HL_ROWS][64]
+  float* xr = hl;
+  float* red = hl + M * K;
+  const int h = blockIdx.y, n = blockIdx.x * 64 + (threadIdx.x & 63), part = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < M * K; i += 256) {
+    const int t = i / K, k = i - t * K;
+    xr[i] = to_f32(x[(long long)t * ldx + (long long)h * xs + k]);
+  }
+  __syncthreads();
+  const int kq = (K + 3) / 4, k0 = part * kq, k1 = min(K, k0 + kq);
+  const T* w = W + ((long long)h * N + min(n, N - 1)) * K;
+  float acc[HL_ROWS];
+#pragma unroll
+  for (int t = 0; t < HL_ROWS; ++t) acc[t] = 0.f;
+  // eight elements of the row of W are asked for before their products (a thread's time is its chain of loads)
+  for (int kb = k0; kb < k1; kb += 8) {
+    float wv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) wv[u] = to_f32(w[min(kb + u, K - 1)]);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int k = kb + u;
+      if (k < k1) {
+#pragma unroll
+        for (int t = 0; t < HL_ROWS; ++t)
+          if (t < M) acc[t] = fmaf(xr[t * K + k], wv[u], acc[t]);
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < HL_ROWS; ++t) red[(part * HL_ROWS + t) * 64 + (threadIdx.x & 63)] = acc[t];
+  __syncthreads();
+  if (n >= N) return;
+  for (int t = part; t < M; t += 4) {
+    float v = 0.f;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) v += red[(p * HL_ROWS + t) * 64 + (threadIdx.x & 63)];
+    if (g) v *= 1.f / (1.f + expf(-to_f32(g[(long long)t * ldg + (long long)h * N + n])));
+    y[(long long)t * ldy + (long long)h * ys + n] = from_f32<T>(v);
+  }
+}
+
 #define DEFINE_LATENT(SUF, T)                                                                              \
   extern "C" int jv_latent_prepare_##SUF(const void* proj, long long ld, int n, int q_rank, int rank,      \
                                          int rot, int rot_dims, const float* wq, const float* wkv,         \
@@ -184,6 +234,12 @@ head_linear_kernel(T* __restrict__ y, long long ldy, int ys, const T* __restrict
     if (M <= 0 || N <= 0 || heads <= 0) return 0;                                                          \
     const unsigned gy = (M + HL_BM - 1) / HL_BM;                                                           \
     if (gy > 65535u || heads > 65535 || K < 0) return (int)hipErrorInvalidValue;                           \
+    if (M <= HL_ROWS && K > 0 && (size_t)(M * K + 4 * HL_ROWS * 64) * sizeof(float) <= 60 * 1024) {        \
+      hipLaunchKernelGGL(head_linear_rows_kernel<T>, dim3((N + 63) / 64, heads), dim3(256),                \
+                         (size_t)(M * K + 4 * HL_ROWS * 64) * sizeof(float), (hipStream_t)stream, (T*)y,   \
+                         ldy, ys, (const T*)x, ldx, xs, (const T*)W, M, N, K, (const T*)g, ldg);           \
+      return JV_LAUNCH_CHECK();                                                                            \
+    }                                                                                                      \
     hipLaunchKernelGGL(head_linear_kernel<T>, dim3((N + HL_BN - 1) / HL_BN, gy, heads), dim3(256), 0,      \
                        (hipStream_t)stream, (T*)y, ldy, ys, (const T*)x, ldx, xs, (const T*)W, M, N, K,    \
                        (const T*)g, ldg);                                                                  \

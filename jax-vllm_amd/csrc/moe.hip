@@ -39,45 +39,82 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int n, int ex
   }
 }
 
-// Router and choice in one launch: one block per token, the token's row in LDS as floats, a wave per
-// expert (in turns) sums its products lane by lane and then across the wave: float logits whatever the
-// activation type, the same order of additions whatever the batch.  logits_out (may be null) [n, experts].
+// Router and choice in one launch: a block takes up to MOE_RT tokens, their rows in LDS as floats; a wave per
+// expert (in turns) reads the expert's router row once and sums its products with every token of the block
+// lane by lane and then across the wave: float logits whatever the activation type, the same order of
+// additions whatever the batch.  Then a wave per token picks the `top` largest, lowest index among equals.
+// logits_out (may be null) [n, experts].
+#define MOE_RT 8
 template <typename T>
 __global__ void __launch_bounds__(256)
-moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, int hidden, int experts, int top,
+moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, int n, int hidden, int experts, int top, int tb,
                   int* __restrict__ ids, float* __restrict__ weights, float* __restrict__ logits_out) {
-  extern __shared__ float rs[];      // x [hidden] | z [experts]
+  extern __shared__ float rs[];      // x [tb][hidden] | z [tb][experts]
   float* xs = rs;
-  float* z = rs + hidden;
-  const long long t = blockIdx.x;
+  float* z = rs + tb * hidden;
+  const long long t0 = (long long)blockIdx.x * tb;
+  const int nt = (int)min((long long)tb, n - t0);
   const int lane = threadIdx.x & (JV_WAVE - 1), wid = threadIdx.x / JV_WAVE, nw = blockDim.x / JV_WAVE;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x) xs[c] = to_f32(x[t * hidden + c]);
+  for (int i = threadIdx.x; i < tb * hidden; i += blockDim.x) {
+    const int t = i / hidden;
+    xs[i] = t < nt ? to_f32(x[t0 * hidden + i]) : 0.f;
+  }
   __syncthreads();
   for (int e = wid; e < experts; e += nw) {
     const T* w = W + (long long)e * hidden;
-    float acc = 0.f;
-    for (int c = lane; c < hidden; c += JV_WAVE) acc = fmaf(xs[c], to_f32(w[c]), acc);
-    acc = wave_sum(acc);
-    if (lane == 0) {
-      z[e] = acc;
-      if (logits_out) logits_out[t * experts + e] = acc;
+    float acc[MOE_RT];
+#pragma unroll
+    for (int t = 0; t < MOE_RT; ++t) acc[t] = 0.f;
+    // eight loads of the router row are asked for before their products: a wave's time here is its chain of loads
+    for (int c0 = lane; c0 < hidden; c0 += 8 * JV_WAVE) {
+      float wv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int c = c0 + u * JV_WAVE;
+        wv[u] = to_f32(w[c < hidden ? c : lane]);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int c = c0 + u * JV_WAVE;
+        if (c < hidden) {
+#pragma unroll
+          for (int t = 0; t < MOE_RT; ++t)
+            if (t < tb) acc[t] = fmaf(xs[t * hidden + c], wv[u], acc[t]);
+        }
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < MOE_RT; ++t) {
+      if (t >= nt) continue;
+      const float v = wave_sum(acc[t]);
+      if (lane == 0) {
+        z[t * experts + e] = v;
+        if (logits_out) logits_out[(t0 + t) * experts + e] = v;
+      }
     }
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
+  for (int t = wid; t < nt; t += nw) {
+    float* zt = z + t * experts;
     for (int kk = 0; kk < top; ++kk) {
-      int best = -1;
-      float bz = -INFINITY;
-      for (int e = 0; e < experts; ++e) {
-        const float v = z[e];
-        if (!(v > bz) && best >= 0) continue;
-        bool taken = false;
-        for (int p = 0; p < kk; ++p) taken |= ids[t * top + p] == e;
-        if (!taken) { best = e; bz = v; }
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+      for (int e = lane; e < experts; e += JV_WAVE) {
+        const float v = zt[e];
+        if (v > bv || (bi == 0x7fffffff && v == v)) { bv = v; bi = e; }
       }
-      if (best < 0) best = 0;
-      ids[t * top + kk] = best;
-      weights[t * top + kk] = 1.f / (1.f + expf(-z[best]));
+#pragma unroll
+      for (int o = JV_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, JV_WAVE);
+        const int oi = __shfl_xor(bi, o, JV_WAVE);
+        if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
+      }
+      if (bi == 0x7fffffff) { bi = kk; bv = __builtin_nanf(""); }      // a row of NaN: some expert, the NaN shows in the output
+      if (lane == 0) {
+        ids[(t0 + t) * top + kk] = bi;
+        weights[(t0 + t) * top + kk] = 1.f / (1.f + expf(-bv));
+      }
+      if ((bi & (JV_WAVE - 1)) == lane) zt[bi] = -INFINITY;      // the lane that scans this expert takes it out
     }
   }
 }
@@ -272,9 +309,12 @@ extern "C" int jv_moe_group(const int* ids, int entries, int experts, int* meta,
     if (n <= 0) return 0;                                                                                         \
     if (experts <= 0 || top <= 0 || top > experts || hidden <= 0 || (hidden + experts) > 15000)                   \
       return (int)hipErrorInvalidValue;                                                                           \
-    hipLaunchKernelGGL(moe_router_kernel<T>, dim3(n), dim3(256), (hidden + experts) * sizeof(float),              \
-                       (hipStream_t)stream, (const T*)x, (const T*)W, hidden, experts, top, ids, weights,         \
-                       logits_out);                                                                               \
+    int tb = 15000 / (hidden + experts);             /* tokens of a block: their rows and logits in 60 KB */      \
+    tb = tb > MOE_RT ? MOE_RT : tb;                                                                               \
+    while (tb > 1 && (n + tb - 1) / tb < 128) --tb;  /* few tokens: more blocks rather than rows sharing a read */ \
+    hipLaunchKernelGGL(moe_router_kernel<T>, dim3((n + tb - 1) / tb), dim3(256),                                  \
+                       (size_t)tb * (hidden + experts) * sizeof(float), (hipStream_t)stream, (const T*)x,         \
+                       (const T*)W, n, hidden, experts, top, tb, ids, weights, logits_out);                       \
     return JV_LAUNCH_CHECK();                                                                                     \
   }                                                                                                               \
   extern "C" int jv_moe_gate_up_##SUF(void* z, const void* x, const void* Wg, const void* Wu, const int* meta,    \

@@ -939,12 +939,35 @@ def lightning_max_dim(chunks: bool) -> int:
     return library.core().jv_lightning_max_dim(c_int(1 if chunks else 0))
 
 
+def lightning_chunk_tokens() -> int:
+    return library.core().jv_lightning_chunk_tokens()
+
+
+def lightning_chunks_possible(dim: int) -> bool:
+    """The kernels by chunks keep a chunk's keys in LDS in 16-byte pieces."""
+    return dim % 4 == 0 and dim <= lightning_max_dim(True)
+
+
+def lightning_chunk_plan(q_lens, device):
+    """(work int32 [chunks, 2] = (request, first token row), first chunk of every request int32 [requests + 1],
+    chunks) for the kernels by chunks: every request's tokens of this step cut into chunks, in order."""
+    size = lightning_chunk_tokens()
+    work, first, at = [], [0], 0
+    for r, n in enumerate(q_lens):
+        work += [(r, at + b) for b in range(0, n, size)]
+        first.append(len(work))
+        at += n
+    flat = torch.tensor([x for w in work for x in w] + first, dtype=torch.int32).pin_memory().to(device, non_blocking=True)
+    return flat[:2 * len(work)], flat[2 * len(work):], len(work)
+
+
 def lightning_attention(proj, q_off: int, k_off: int, v_off: int, state, slot_ids, cu_seqlens, decay, heads: int,
-                        dim: int, vdim: int, chunks: bool) -> torch.Tensor:
+                        dim: int, vdim: int, chunk_plan=None) -> torch.Tensor:
     """Float [n, heads * vdim]: o_t = S_t^T q_t with S_t = decay_h S_(t-1) + k_t v_t^T per request and head,
     q, k, v = silu of the columns of ``proj`` at the given offsets (head by head).  ``state``
     [slots + 1, heads, dim, vdim] float holds S of every request before the step and after it.
-    ``chunks``: the kernel that takes a request's tokens 32 at a time instead of one by one."""
+    ``chunk_plan`` (``lightning_chunk_plan`` of the step's token counts): the kernels that take a request's
+    tokens a chunk at a time, chunks side by side, instead of one by one."""
     _dev(proj, state, slot_ids, cu_seqlens, decay)
     n, ld = proj.shape
     r = slot_ids.numel()
@@ -954,12 +977,21 @@ def lightning_attention(proj, q_off: int, k_off: int, v_off: int, state, slot_id
     _f32(state, "state")
     _need(state.dim() == 4 and tuple(state.shape[1:]) == (heads, dim, vdim), "state must be [slots, heads, dim, vdim]")
     _need(max(q_off, k_off) + heads * dim <= ld and v_off + heads * vdim <= ld, "proj rows are too short")
-    _need(dim <= lightning_max_dim(chunks), f"key size {dim} above the kernel's {lightning_max_dim(chunks)}")
+    _need(dim <= lightning_max_dim(False), f"key size {dim} above the kernel's {lightning_max_dim(False)}")
     out = torch.empty((n, heads * vdim), dtype=torch.float32, device=proj.device)
+    work = first = scratch = None
+    chunks = 0
+    if chunk_plan is not None:
+        work, first, chunks = chunk_plan
+        _need(lightning_chunks_possible(dim), "the kernels by chunks take key sizes that are multiples of 4, at most 128")
+        _dev(work, first)
+        _i32(work, "work", 2 * chunks)
+        _i32(first, "first chunks", r + 1)
+        scratch = torch.empty(chunks * heads * dim * vdim, dtype=torch.float32, device=proj.device)
     fn = getattr(library.core(), f"jv_lightning_{_suffix(proj.dtype)}")
     _check(fn(_ptr(out), _ptr(proj), c_longlong(ld), c_int(q_off), c_int(k_off), c_int(v_off), _ptr(state),
               _ptr(slot_ids), _ptr(cu_seqlens), _ptr(decay), c_int(r), c_int(heads), c_int(dim), c_int(vdim),
-              c_int(1 if chunks else 0), _stream()), "lightning_attention")
+              c_int(chunks), _ptr(work), _ptr(first), _ptr(scratch), _stream()), "lightning_attention")
     return out
 
 
@@ -1019,11 +1051,17 @@ def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, lo
     return MoePlan(ids, weights, meta, offsets, tile_expert, tile_row0, order, max_tiles, top)
 
 
+def moe_matrix_cores_possible(dtype, hidden: int, ff: int) -> bool:
+    """The grouped products have a matrix-core form for bfloat16 and inner sizes that are multiples of 8."""
+    return dtype == torch.bfloat16 and hidden % 8 == 0 and ff % 8 == 0 and hidden >= 8 and ff >= 8
+
+
 def moe_experts(x, plan: MoePlan, w_gate, w_up, w_down, activation: str, out: torch.Tensor,
-                weight_on_input: bool = True) -> None:
+                weight_on_input: bool = True, matrix_cores: "bool | None" = None) -> None:
     """out[kk, t] = down[e] (act(gate[e] xs) * (up[e] xs)) for the kk-th chosen expert e of token t, float32
     [top, n, hidden]; xs = weight * x[t] with ``weight_on_input``, else x[t] and the result is multiplied
-    by the weight.  w_gate, w_up [experts, ff, hidden], w_down [experts, hidden, ff]."""
+    by the weight.  w_gate, w_up [experts, ff, hidden], w_down [experts, hidden, ff].  ``matrix_cores``:
+    None takes the matrix-core kernels wherever ``moe_matrix_cores_possible``, False the float-FMA ones."""
     _dev(x, w_gate, w_up, w_down, out)
     n, hidden = x.shape
     experts, ff, _ = w_gate.shape
@@ -1034,6 +1072,10 @@ def moe_experts(x, plan: MoePlan, w_gate, w_up, w_down, activation: str, out: to
     _need(plan.ids.numel() == n * plan.top, "the plan belongs to another step")
     z = torch.empty((n * plan.top, ff), dtype=x.dtype, device=x.device)
     lib, suf = library.core(), _suffix(x.dtype)
+    possible = moe_matrix_cores_possible(x.dtype, hidden, ff)
+    _need(not matrix_cores or possible, "the matrix-core kernels take bfloat16 and inner sizes that are multiples of 8")
+    if possible and matrix_cores is not False:
+        suf = "mfma_bf16"
     p = plan
     _check(getattr(lib, f"jv_moe_gate_up_{suf}")(
         _ptr(z), _ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(p.meta), _ptr(p.offsets), _ptr(p.tile_expert),

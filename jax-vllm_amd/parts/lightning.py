@@ -55,9 +55,14 @@ class LightningAttention:
     def forward(self, x, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
         H, d, dv = self.heads, self.dim, self.vdim
         proj = K.linear(x, self.w_in)
-        chunks = ctx.max_q_len >= K.LIGHTNING_CHUNK_MIN_TOKENS and d <= K.lightning_max_dim(True)
+        plan = None
+        if not ctx.captured and ctx.max_q_len >= K.LIGHTNING_CHUNK_MIN_TOKENS and K.lightning_chunks_possible(d):
+            # prompt portions: chunks side by side (the list of chunks is the same for every such layer of the step)
+            plan = ctx.plans.get("lightning_chunks")
+            if plan is None:
+                plan = ctx.plans["lightning_chunks"] = K.lightning_chunk_plan(ctx.q_lens_host, x.device)
         o = K.lightning_attention(proj, 0, H * d, 2 * H * d, mem.state, ctx.slot_ids, ctx.cu_seqlens, self.decay,
-                                  H, d, dv, chunks)
+                                  H, d, dv, plan)
         y = K.gated_rmsnorm(o, proj[:, 2 * H * d + H * dv:], self.norm_weight, self.eps)
         return K.linear(y, self.w_o, partial_ok=True)
 

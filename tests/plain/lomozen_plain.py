@@ -49,9 +49,31 @@ def silu(z):
     return z * torch.sigmoid(z)
 
 
+_ROUND_PRODUCTS_TO = None     # see ``rounded_products``
+
+
 def linear(x, w):
     """w is stored [out, in]."""
-    return x @ w.T
+    y = x @ w.T
+    return y if _ROUND_PRODUCTS_TO is None else y.to(_ROUND_PRODUCTS_TO).to(y.dtype)
+
+
+class rounded_products:
+    """Within this context every matrix product's result is rounded to ``dtype`` (and widened again): what
+    an implementation that keeps its activations in bfloat16 does to the numbers at the least.  The
+    difference to the unrounded run says how much of such rounding the model at hand lets through to its
+    logits, which is the measure for the bfloat16 tests' tolerances."""
+
+    def __init__(self, dtype=torch.bfloat16):
+        self.dtype = dtype
+
+    def __enter__(self):
+        global _ROUND_PRODUCTS_TO
+        self.before, _ROUND_PRODUCTS_TO = _ROUND_PRODUCTS_TO, self.dtype
+
+    def __exit__(self, *exc):
+        global _ROUND_PRODUCTS_TO
+        _ROUND_PRODUCTS_TO = self.before
 
 
 # --------------------------------------------------------------------------- rotation
