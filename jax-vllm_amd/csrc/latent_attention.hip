@@ -206,6 +206,53 @@ head_linear_rows_kernel(T* __restrict__ y, long long ldy, int ys, const T* __res
   }
 }
 
+// The same on the matrix cores (bfloat16; K, the head strides and the row strides multiples of 8): a wave takes
+// 16 outputs of one head against 16 rows, both operands straight from global memory in 16-byte pieces
+// (v_mfma_f32_16x16x32_bf16, A = 16 rows of W, B = 16 rows of x; the accumulator holds y^T[n = 4 lc + e][m = li]);
+// the 4 waves of a block take 4 row tiles against the same 16 rows of W.  grid (N / 16, M / 64, heads).
+typedef __bf16 hl_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float hl_f32x4 __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256)
+head_linear_mfma_kernel(bf16_t* __restrict__ y, long long ldy, int ys, const bf16_t* __restrict__ x, long long ldx,
+                        int xs, const bf16_t* __restrict__ W, int M, int N, int K, const bf16_t* __restrict__ g,
+                        long long ldg) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, li = lane & 15, lc = lane >> 4;
+  const int h = blockIdx.z, n0 = blockIdx.x * 16, m0 = (blockIdx.y * 4 + wave) * 16;
+  if (m0 >= M) return;
+  const bf16_t* wr = W + ((long long)h * N + min(n0 + li, N - 1)) * K;
+  const bf16_t* xr = x + (long long)min(m0 + li, M - 1) * ldx + (long long)h * xs;
+  const hl_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  hl_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 64) {        // two steps a turn: four loads asked for before the products
+    const int ka = k0 + lc * 8, kb = ka + 32;
+    const hl_bf16x8 a0 = *(const hl_bf16x8*)(wr + min(ka, K - 8)), b0 = *(const hl_bf16x8*)(xr + min(ka, K - 8));
+    const hl_bf16x8 a1 = *(const hl_bf16x8*)(wr + min(kb, K - 8)), b1 = *(const hl_bf16x8*)(xr + min(kb, K - 8));
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, ka < K ? b0 : zero, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, kb < K ? b1 : zero, acc, 0, 0, 0);
+  }
+  const int m = m0 + li, nb = n0 + lc * 4;
+  if (m >= M) return;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int n = nb + e;
+    if (n >= N) continue;
+    float v = acc[e];
+    if (g) v *= 1.f / (1.f + expf(-(float)g[(long long)m * ldg + (long long)h * N + n]));
+    y[(long long)m * ldy + (long long)h * ys + n] = (bf16_t)v;
+  }
+}
+
+extern "C" int jv_head_linear_mfma_bf16(void* y, long long ldy, int ys, const void* x, long long ldx, int xs,
+                                        const void* W, int M, int N, int K, int heads, const void* g, long long ldg,
+                                        void* stream) {
+  if (M <= 0 || N <= 0 || heads <= 0) return 0;
+  const unsigned gy = (M + 63) / 64;
+  if (gy > 65535u || heads > 65535 || K < 8 || K % 8 || ldx % 8 || xs % 8) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(head_linear_mfma_kernel, dim3((N + 15) / 16, gy, heads), dim3(256), 0, (hipStream_t)stream,
+                     (bf16_t*)y, ldy, ys, (const bf16_t*)x, ldx, xs, (const bf16_t*)W, M, N, K, (const bf16_t*)g, ldg);
+  return JV_LAUNCH_CHECK();
+}
+
 #define DEFINE_LATENT(SUF, T)                                                                              \
   extern "C" int jv_latent_prepare_##SUF(const void* proj, long long ld, int n, int q_rank, int rank,      \
                                          int rot, int rot_dims, const float* wq, const float* wkv,         \

@@ -17,26 +17,42 @@
 #define MOE_TN 64
 #define MOE_BK 16
 
-// one thread per token
-__global__ void moe_route_kernel(const float* __restrict__ logits, int n, int experts, int top,
-                                 int* __restrict__ ids, float* __restrict__ weights) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n) return;
-  const float* z = logits + (long long)t * experts;
+// The `top` largest of a token's logits, lowest index among equals: the lanes of a wave scan the token's
+// logits (a copy in LDS), the wave agrees on the best, and the lane that scans the chosen expert takes it out.
+__device__ __forceinline__ void moe_pick(float* zt, int experts, int top, int lane, int* ids, float* weights) {
   for (int kk = 0; kk < top; ++kk) {
-    int best = -1;
-    float bz = -INFINITY;
-    for (int e = 0; e < experts; ++e) {
-      const float v = z[e];
-      if (!(v > bz) && best >= 0) continue;
-      bool taken = false;
-      for (int p = 0; p < kk; ++p) taken |= ids[(long long)t * top + p] == e;
-      if (!taken) { best = e; bz = v; }
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < experts; e += JV_WAVE) {
+      const float v = zt[e];
+      if (v > bv || (bi == 0x7fffffff && v == v)) { bv = v; bi = e; }
     }
-    if (best < 0) best = 0;        // rows of NaN: some expert, the NaN shows in the output
-    ids[(long long)t * top + kk] = best;
-    weights[(long long)t * top + kk] = 1.f / (1.f + expf(-z[best]));
+#pragma unroll
+    for (int o = JV_WAVE / 2; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, JV_WAVE);
+      const int oi = __shfl_xor(bi, o, JV_WAVE);
+      if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
+    }
+    if (bi == 0x7fffffff) { bi = kk; bv = __builtin_nanf(""); }      // a row of NaN: some expert, the NaN shows in the output
+    if (lane == 0) {
+      ids[kk] = bi;
+      weights[kk] = 1.f / (1.f + expf(-bv));
+    }
+    if ((bi & (JV_WAVE - 1)) == lane) zt[bi] = -INFINITY;
   }
+}
+
+// a wave per token, 4 tokens a block
+__global__ void __launch_bounds__(256)
+moe_route_kernel(const float* __restrict__ logits, int n, int experts, int top,
+                 int* __restrict__ ids, float* __restrict__ weights) {
+  extern __shared__ float zs[];      // [4][experts]
+  const int lane = threadIdx.x & (JV_WAVE - 1), wid = threadIdx.x / JV_WAVE;
+  const long long t = (long long)blockIdx.x * 4 + wid;
+  if (t >= n) return;
+  float* zt = zs + wid * experts;
+  for (int e = lane; e < experts; e += JV_WAVE) zt[e] = logits[t * experts + e];
+  moe_pick(zt, experts, top, lane, ids + t * top, weights + t * top);
 }
 
 // Router and choice in one launch: a block takes up to MOE_RT tokens, their rows in LDS as floats; a wave per
@@ -46,7 +62,7 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int n, int ex
 // logits_out (may be null) [n, experts].
 #define MOE_RT 8
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, int n, int hidden, int experts, int top, int tb,
                   int* __restrict__ ids, float* __restrict__ weights, float* __restrict__ logits_out) {
   extern __shared__ float rs[];      // x [tb][hidden] | z [tb][experts]
@@ -94,35 +110,14 @@ moe_router_kernel(const T* __restrict__ x, const T* __restrict__ W, int n, int h
     }
   }
   __syncthreads();
-  for (int t = wid; t < nt; t += nw) {
-    float* zt = z + t * experts;
-    for (int kk = 0; kk < top; ++kk) {
-      float bv = -INFINITY;
-      int bi = 0x7fffffff;
-      for (int e = lane; e < experts; e += JV_WAVE) {
-        const float v = zt[e];
-        if (v > bv || (bi == 0x7fffffff && v == v)) { bv = v; bi = e; }
-      }
-#pragma unroll
-      for (int o = JV_WAVE / 2; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(bv, o, JV_WAVE);
-        const int oi = __shfl_xor(bi, o, JV_WAVE);
-        if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
-      }
-      if (bi == 0x7fffffff) { bi = kk; bv = __builtin_nanf(""); }      // a row of NaN: some expert, the NaN shows in the output
-      if (lane == 0) {
-        ids[(t0 + t) * top + kk] = bi;
-        weights[(t0 + t) * top + kk] = 1.f / (1.f + expf(-bv));
-      }
-      if ((bi & (JV_WAVE - 1)) == lane) zt[bi] = -INFINITY;      // the lane that scans this expert takes it out
-    }
-  }
+  for (int t = wid; t < nt; t += nw)
+    moe_pick(z + t * experts, experts, top, lane, ids + (t0 + t) * top, weights + (t0 + t) * top);
 }
 
 // One block.  meta: [0] number of tiles; offsets [experts + 1]; tile_expert / tile_row0 [max_tiles];
-// order [entries]: entry index at each position; rank [entries] scratch.
+// order [entries]: entry index at each position; rank [entries] scratch.  A tile has tile_rows rows.
 __global__ void __launch_bounds__(1024)
-moe_group_kernel(const int* __restrict__ ids, int entries, int experts, int* __restrict__ meta,
+moe_group_kernel(const int* __restrict__ ids, int entries, int experts, int tile_rows, int* __restrict__ meta,
                  int* __restrict__ offsets, int* __restrict__ tile_expert, int* __restrict__ tile_row0,
                  int* __restrict__ order, int* __restrict__ rank) {
   extern __shared__ int sh[];      // count [experts] | start [experts + 1] | first tile [experts + 1]
@@ -139,7 +134,7 @@ moe_group_kernel(const int* __restrict__ ids, int entries, int experts, int* __r
       start[e] = at;
       tile0[e] = tiles;
       at += count[e];
-      tiles += (count[e] + MOE_TM - 1) / MOE_TM;
+      tiles += (count[e] + tile_rows - 1) / tile_rows;
     }
     start[experts] = at;
     tile0[experts] = tiles;
@@ -150,7 +145,7 @@ moe_group_kernel(const int* __restrict__ ids, int entries, int experts, int* __r
   for (int e = threadIdx.x; e < experts; e += blockDim.x)
     for (int i = tile0[e]; i < tile0[e + 1]; ++i) {
       tile_expert[i] = e;
-      tile_row0[i] = start[e] + (i - tile0[e]) * MOE_TM;
+      tile_row0[i] = start[e] + (i - tile0[e]) * tile_rows;
     }
   for (int s = threadIdx.x; s < entries; s += blockDim.x) order[start[ids[s]] + rank[s]] = s;
 }
@@ -289,17 +284,18 @@ extern "C" int jv_moe_tile_rows() { return MOE_TM; }
 extern "C" int jv_moe_route(const float* logits, int n, int experts, int top, int* ids, float* weights, void* stream) {
   if (n <= 0) return 0;
   if (experts <= 0 || top <= 0 || top > experts) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(moe_route_kernel, dim3((n + 127) / 128), dim3(128), 0, (hipStream_t)stream, logits, n, experts,
-                     top, ids, weights);
+  if (experts > 3840) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((n + 3) / 4), dim3(256), 4 * experts * sizeof(float), (hipStream_t)stream,
+                     logits, n, experts, top, ids, weights);
   return JV_LAUNCH_CHECK();
 }
 
-extern "C" int jv_moe_group(const int* ids, int entries, int experts, int* meta, int* offsets, int* tile_expert,
-                            int* tile_row0, int* order, int* rank, void* stream) {
+extern "C" int jv_moe_group(const int* ids, int entries, int experts, int tile_rows, int* meta, int* offsets,
+                            int* tile_expert, int* tile_row0, int* order, int* rank, void* stream) {
   if (entries <= 0) return 0;
-  if (experts <= 0 || experts > 4096) return (int)hipErrorInvalidValue;
+  if (experts <= 0 || experts > 4096 || tile_rows <= 0) return (int)hipErrorInvalidValue;
   hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (3 * experts + 2) * sizeof(int), (hipStream_t)stream, ids,
-                     entries, experts, meta, offsets, tile_expert, tile_row0, order, rank);
+                     entries, experts, tile_rows, meta, offsets, tile_expert, tile_row0, order, rank);
   return JV_LAUNCH_CHECK();
 }
 
@@ -312,7 +308,7 @@ extern "C" int jv_moe_group(const int* ids, int entries, int experts, int* meta,
     int tb = 15000 / (hidden + experts);             /* tokens of a block: their rows and logits in 60 KB */      \
     tb = tb > MOE_RT ? MOE_RT : tb;                                                                               \
     while (tb > 1 && (n + tb - 1) / tb < 128) --tb;  /* few tokens: more blocks rather than rows sharing a read */ \
-    hipLaunchKernelGGL(moe_router_kernel<T>, dim3((n + tb - 1) / tb), dim3(256),                                  \
+    hipLaunchKernelGGL(moe_router_kernel<T>, dim3((n + tb - 1) / tb), dim3(1024),                                  \
                        (size_t)tb * (hidden + experts) * sizeof(float), (hipStream_t)stream, (const T*)x,         \
                        (const T*)W, n, hidden, experts, top, tb, ids, weights, logits_out);                       \
     return JV_LAUNCH_CHECK();                                                                                     \

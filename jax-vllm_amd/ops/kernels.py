@@ -911,10 +911,12 @@ def latent_query_rope(q, qe, heads: int, dim: int, rot: int, rot_dims: int, rank
               _ptr(cos_sin), _stream()), "latent_query_rope")
 
 
-def head_linear(y, y_head_stride: int, x, x_head_stride: int, w, gate=None) -> None:
+def head_linear(y, y_head_stride: int, x, x_head_stride: int, w, gate=None, matrix_cores: "bool | None" = None) -> None:
     """One matrix per head: y[t, h * ys : h * ys + N] = w[h] @ x[t, h * xs : h * xs + K], w [heads, N, K];
     with ``gate`` (a [n, heads * N] view with unit column stride) the result is multiplied by sigmoid(gate).
-    x and y are row-major matrices of the activation type; float accumulation."""
+    x and y are row-major matrices of the activation type; float accumulation.  bfloat16 with K, the row
+    stride and the head stride of x multiples of 8 runs on the matrix cores (``matrix_cores`` False: the
+    float-FMA kernels all the same)."""
     _dev(y, x, w)
     heads, N, K = w.shape
     n = x.shape[0]
@@ -925,7 +927,11 @@ def head_linear(y, y_head_stride: int, x, x_head_stride: int, w, gate=None) -> N
     if gate is not None:
         _need(gate.is_cuda and gate.dtype == x.dtype and gate.shape == (n, heads * N) and gate.stride(1) == 1,
               "gate must be a [n, heads * N] view with unit column stride")
-    fn = getattr(library.core(), f"jv_head_linear_{_suffix(x.dtype)}")
+    possible = (x.dtype == torch.bfloat16 and K >= 8 and K % 8 == 0 and x.shape[1] % 8 == 0 and x_head_stride % 8 == 0
+                and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+    _need(not matrix_cores or possible, "the matrix-core kernel takes bfloat16 and sizes and strides that are multiples of 8")
+    name = "jv_head_linear_mfma_bf16" if possible and matrix_cores is not False else f"jv_head_linear_{_suffix(x.dtype)}"
+    fn = getattr(library.core(), name)
     _check(fn(_ptr(y), c_longlong(y.shape[1]), c_int(y_head_stride), _ptr(x), c_longlong(x.shape[1]),
               c_int(x_head_stride), _ptr(w), c_int(n), c_int(N), c_int(K), c_int(heads), _ptr(gate),
               c_longlong(0 if gate is None else gate.stride(0)), _stream()), "head_linear")
@@ -997,23 +1003,62 @@ def lightning_attention(proj, q_off: int, k_off: int, v_off: int, state, slot_id
 
 # --------------------------------------------------------------------------- routed experts
 def moe_tile_rows() -> int:
+    """Rows of a tile of the float-FMA expert kernels (the matrix-core ones also take tiles of 128)."""
     return library.core().jv_moe_tile_rows()
+
+
+def moe_tile_rows_for(dtype, hidden: int, ff: int, entries: int, experts: int) -> int:
+    """Rows of a tile for a step: 128 where the matrix-core kernels run and an expert gets about a
+    hundred rows or more (a row of W then feeds twice the products), else 64."""
+    if moe_matrix_cores_possible(dtype, hidden, ff) and entries >= 96 * experts:
+        return 128
+    return moe_tile_rows()
+
+
+def gemm_rows_f32out(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """float32 x @ w.T for bfloat16 x [M, K] and w [N, K] on the matrix cores (K a multiple of 8): products
+    whose result must not be rounded to the activation type (router logits)."""
+    _dev(x, w)
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_rows_f32out takes bfloat16")
+    m, k = x.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k and k % 8 == 0 and k >= 8, "inner sizes must agree and be a multiple of 8")
+    out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    _check(library.core().jv_gemm_rows_f32out_bf16(_ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), _stream()),
+           "gemm_rows_f32out")
+    return out
 
 
 class MoePlan:
     """Device-side grouping of a step's (token, choice) entries by expert."""
 
-    def __init__(self, ids, weights, meta, offsets, tile_expert, tile_row0, order, max_tiles, top):
+    def __init__(self, ids, weights, meta, offsets, tile_expert, tile_row0, order, max_tiles, top, tile_rows):
         self.ids, self.weights, self.meta, self.offsets = ids, weights, meta, offsets
         self.tile_expert, self.tile_row0, self.order, self.max_tiles, self.top = tile_expert, tile_row0, order, max_tiles, top
+        self.tile_rows = tile_rows
 
 
-def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, logits_out=None) -> MoePlan:
+def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, logits_out=None,
+              tile_rows: "int | None" = None) -> MoePlan:
     """Chooses for every token the ``top`` experts with the largest router logits (weights sigmoid(logit);
     the lowest index among equal logits) and orders the n * top entries by expert, all on the device.
     Either float ``logits`` [n, experts] are given, or rows ``x`` [n, hidden] and the router matrix
-    ``w_router`` [experts, hidden] of one type: then the logits are made in the same launch, in float
-    (``logits_out``, float32 [n, experts], receives them if given)."""
+    ``w_router`` [experts, hidden] of one type: then the logits are made here, in float (``logits_out``,
+    float32 [n, experts], receives them if given): in the same launch as the choice (float32, odd sizes), or
+    for bfloat16 by a matrix-core product with float output before it.  ``tile_rows``: rows of a tile of the grouping
+    (``moe_tile_rows_for``; default: the float-FMA kernels' 64)."""
+    if (logits is None and x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and x.shape[1] >= 8
+            and w_router.shape[0] <= 3840):
+        # bfloat16: the logits come from a matrix-core product with float output (never rounded to bfloat16): the
+        # weight-streaming one for the few rows of a decode step, the tiled one for more
+        rows = x.shape[0]
+        plan = streaming_plan(rows, w_router.shape[0], w_router.shape[1], device=x.device) if rows <= SKINNY_AUTO_ROWS else None
+        if plan is not None and plan[1] == 1:
+            logits = gemm_skinny(x, w_router, torch.float32, block_shape=plan[0])
+        else:
+            logits = gemm_rows_f32out(x, w_router)
+        if logits_out is not None:
+            logits_out.copy_(logits)
     if logits is not None:
         _dev(logits)
         _f32(logits, "logits")
@@ -1030,7 +1075,9 @@ def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, lo
         dev = x.device
     _need(0 < top <= experts, "top must be between 1 and the number of experts")
     entries = n * top
-    max_tiles = -(-entries // moe_tile_rows()) + experts
+    tile_rows = tile_rows or moe_tile_rows()
+    _need(tile_rows in (64, 128), "tiles have 64 or 128 rows")
+    max_tiles = -(-entries // tile_rows) + experts
     ints = torch.empty(entries * 3 + 1 + experts + 1 + 2 * max_tiles, dtype=torch.int32, device=dev)
     ids, rank, order = ints[:entries], ints[entries:2 * entries], ints[2 * entries:3 * entries]
     at = 3 * entries
@@ -1046,9 +1093,9 @@ def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, lo
         _check(getattr(lib, f"jv_moe_router_{_suffix(x.dtype)}")(
             _ptr(x), _ptr(w_router), c_int(n), c_int(hidden), c_int(experts), c_int(top), _ptr(ids), _ptr(weights),
             _ptr(logits_out), _stream()), "moe_router")
-    _check(lib.jv_moe_group(_ptr(ids), c_int(entries), c_int(experts), _ptr(meta), _ptr(offsets), _ptr(tile_expert),
+    _check(lib.jv_moe_group(_ptr(ids), c_int(entries), c_int(experts), c_int(tile_rows), _ptr(meta), _ptr(offsets), _ptr(tile_expert),
                             _ptr(tile_row0), _ptr(order), _ptr(rank), _stream()), "moe_group")
-    return MoePlan(ids, weights, meta, offsets, tile_expert, tile_row0, order, max_tiles, top)
+    return MoePlan(ids, weights, meta, offsets, tile_expert, tile_row0, order, max_tiles, top, tile_rows)
 
 
 def moe_matrix_cores_possible(dtype, hidden: int, ff: int) -> bool:
@@ -1074,9 +1121,19 @@ def moe_experts(x, plan: MoePlan, w_gate, w_up, w_down, activation: str, out: to
     lib, suf = library.core(), _suffix(x.dtype)
     possible = moe_matrix_cores_possible(x.dtype, hidden, ff)
     _need(not matrix_cores or possible, "the matrix-core kernels take bfloat16 and inner sizes that are multiples of 8")
-    if possible and matrix_cores is not False:
-        suf = "mfma_bf16"
+    mfma = possible and matrix_cores is not False
+    _need(mfma or plan.tile_rows == moe_tile_rows(), "the float-FMA kernels take tiles of 64 rows")
     p = plan
+    if mfma:
+        _check(lib.jv_moe_gate_up_mfma_bf16(
+            _ptr(z), _ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(p.meta), _ptr(p.offsets), _ptr(p.tile_expert),
+            _ptr(p.tile_row0), _ptr(p.order), _ptr(p.weights), c_int(p.max_tiles), c_int(p.top), c_int(hidden), c_int(ff),
+            c_int(_gate_act_id(activation)), c_int(1 if weight_on_input else 0), c_int(p.tile_rows), _stream()), "moe_gate_up")
+        _check(lib.jv_moe_down_mfma_bf16(
+            _ptr(out), _ptr(z), _ptr(w_down), _ptr(p.meta), _ptr(p.offsets), _ptr(p.tile_expert), _ptr(p.tile_row0),
+            _ptr(p.order), _ptr(p.weights), c_int(p.max_tiles), c_int(p.top), c_int(n), c_int(hidden), c_int(ff),
+            c_int(0 if weight_on_input else 1), c_int(p.tile_rows), _stream()), "moe_down")
+        return
     _check(getattr(lib, f"jv_moe_gate_up_{suf}")(
         _ptr(z), _ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(p.meta), _ptr(p.offsets), _ptr(p.tile_expert),
         _ptr(p.tile_row0), _ptr(p.order), _ptr(p.weights), c_int(p.max_tiles), c_int(p.top), c_int(hidden), c_int(ff),

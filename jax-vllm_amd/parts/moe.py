@@ -63,7 +63,8 @@ class RoutedExperts:
 
     def forward(self, x, ctx=None):
         n = x.shape[0]
-        plan = K.moe_route(None, self.top, x=x, w_router=self.w_router)
+        plan = K.moe_route(None, self.top, x=x, w_router=self.w_router,
+                           tile_rows=K.moe_tile_rows_for(x.dtype, self.hidden_size, self.ff, n * self.top, self.experts))
         out = torch.empty((self.top, n, self.hidden_size), dtype=torch.float32, device=x.device)
         K.moe_experts(x, plan, self.w_gate, self.w_up, self.w_down, self.activation, out, self.weight_on_input)
         rows = self.shared.forward(x, ctx) if self.shared is not None else None

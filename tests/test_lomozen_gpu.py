@@ -326,7 +326,8 @@ def test_routed_expert_kernels(dtype, n, experts, top, hidden, ff):
     srt = torch.sort(z, dim=-1, descending=True).values
     clear = torch.ones(n, dtype=torch.bool) if top == experts else (srt[:, top - 1] - srt[:, top]) > 1e-3
     logits = torch.empty(n, experts, dtype=torch.float32, device="cuda")
-    plan = K.moe_route(None, top, x=x.cuda(), w_router=wr.cuda(), logits_out=logits)
+    tile_rows = 128 if (n >= 100 and K.moe_matrix_cores_possible(dtype, hidden, ff)) else None
+    plan = K.moe_route(None, top, x=x.cuda(), w_router=wr.cuda(), logits_out=logits, tile_rows=tile_rows)
     assert float((logits.cpu().double() - z).abs().max()) <= 1e-5 * float(z.abs().max())
     ids = plan.ids.cpu().view(n, top).long()
     want_ids = torch.topk(z, top, dim=-1).indices
@@ -335,7 +336,9 @@ def test_routed_expert_kernels(dtype, n, experts, top, hidden, ff):
     assert sorted(order.tolist()) == list(range(n * top)) and int(offsets[-1]) == n * top
     for e in range(experts):
         assert (plan.ids.cpu()[order[offsets[e]:offsets[e + 1]]] == e).all()
-    forms = [None, False] if K.moe_matrix_cores_possible(dtype, hidden, ff) else [None]     # matrix cores and float FMA
+    again = K.moe_route(logits, top)                       # the choice from given logits is the same choice
+    assert torch.equal(again.ids, plan.ids) and torch.equal(again.weights, plan.weights)
+    forms = [None, False] if K.moe_matrix_cores_possible(dtype, hidden, ff) and not tile_rows else [None]     # matrix cores and float FMA
     for on_input, form in [(a, b) for a in (True, False) for b in forms]:
         out = torch.full((top, n, hidden), float("nan"), dtype=torch.float32, device="cuda")
         K.moe_experts(x.cuda(), plan, wg.cuda(), wu.cuda(), wd.cuda(), "silu", out, weight_on_input=on_input,
@@ -384,3 +387,28 @@ def test_norm_of_a_sublayer_output_joined_to_the_stream(dtype):
                                w.cuda(), out, rows, out_eps=1e-5)
         assert torch.equal(h.cpu(), h0)
         assert float((out.cpu().double() - want[[7, 0, 3]]).abs().max()) <= (1e-5 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("n,heads,N,K", [(1, 3, 24, 16), (9, 2, 40, 72), (70, 5, 20, 24), (200, 2, 100, 136), (5, 4, 7, 10)])
+def test_one_matrix_per_head(dtype, n, heads, N, K):
+    """Every form of the per-head product (few rows, tiles, matrix cores) against float64, with heads that sit at
+    strides wider than their sizes, with and without the sigmoid gate."""
+    from jax_vllm_amd.ops import kernels as K_
+
+    g = torch.Generator().manual_seed(n + N)
+    xs, ys = K + 8, N + 3
+    x = torch.randn(n, heads * xs, generator=g).to(dtype)
+    w = (torch.randn(heads, N, K, generator=g) * K ** -0.5).to(dtype)
+    gate = torch.randn(n, heads * N + 5, generator=g).to(dtype)
+    want = torch.einsum("hnk,thk->thn", w.double(), x.double().view(n, heads, xs)[..., :K])
+    forms = [None, False] if dtype == torch.bfloat16 and K % 8 == 0 else [None]
+    for gated, form in [(a, b) for a in (False, True) for b in forms]:
+        y = torch.zeros(n, heads * ys, dtype=dtype, device="cuda")
+        gv = gate.cuda()[:, 5:] if gated else None
+        K_.head_linear(y, ys, x.cuda(), xs, w.cuda(), gate=gv, matrix_cores=form)
+        ref = want * torch.sigmoid(gate.double()[:, 5:].view(n, heads, N)) if gated else want
+        got = y.cpu().double().view(n, heads, ys)
+        tol = 1e-5 if dtype == torch.float32 else 1e-2
+        assert float((got[..., :N] - ref).abs().max()) <= tol * max(1.0, float(ref.abs().max())), f"gated={gated} form={form}"
+        assert float(got[..., N:].abs().max()) == 0.0           # nothing is written between the heads
