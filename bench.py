@@ -2,6 +2,7 @@
 prefill tokens/s at 2,048 tokens and decode at batch 1 and 64 beside it.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--shape 8b|14b|32b]
+    python bench.py --only design [--design-shape 2k|4k]     # the Lomozen architecture beside the dense model of equal size
 
 The model has the layer sizes of Qwen3-8B (the headline configuration) with random
 weights drawn on the device; prompts are seeded uniform-random token ids of 1,024 tokens;

@@ -1,4 +1,4 @@
-"""MI355X-native Qwen3 inference engine (import name ``jax_vllm_amd``)."""
+"""MI355X-native inference engine for Qwen3 dense and Lomozen (import name ``jax_vllm_amd``)."""
 from .config import ConfigError, EngineConfig
 from .engine.request import EngineStats, Request, SamplingParams, StepEvent
 

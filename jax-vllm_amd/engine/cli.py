@@ -20,7 +20,7 @@ import sys
 
 
 def build_parser() -> argparse.ArgumentParser:
-    p = argparse.ArgumentParser(prog="jax_vllm_amd", description="Generate token ids with the MI355X Qwen3 engine.")
+    p = argparse.ArgumentParser(prog="jax_vllm_amd", description="Generate token ids with the MI355X engine (Qwen3 dense, Lomozen).")
     p.add_argument("--model-path", default=os.environ.get("JLLM_MODEL_PATH"),
                    help="Path to HF model directory (config.json + *.safetensors). Env: JLLM_MODEL_PATH.")
     p.add_argument("--max-num-seqs", type=int, default=4)

@@ -1015,6 +1015,9 @@ def moe_tile_rows_for(dtype, hidden: int, ff: int, entries: int, experts: int) -
     return moe_tile_rows()
 
 
+ROUTER_FUSED_MAX_ROWS = 64      # 17..64 rows: logits and choice in one launch
+
+
 def gemm_rows_f32out(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """float32 x @ w.T for bfloat16 x [M, K] and w [N, K] on the matrix cores (K a multiple of 8): products
     whose result must not be rounded to the activation type (router logits)."""
@@ -1050,14 +1053,15 @@ def moe_route(logits: "torch.Tensor | None", top: int, x=None, w_router=None, lo
     if (logits is None and x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0 and x.shape[1] >= 8
             and w_router.shape[0] <= 3840):
         # bfloat16: the logits come from a matrix-core product with float output (never rounded to bfloat16): the
-        # weight-streaming one for the few rows of a decode step, the tiled one for more
+        # weight-streaming one for the few rows of a decode step, the tiled one for prompt portions; between
+        # them (measured at 32 rows: one block of the tiled product walks the whole router alone) the fused kernel
         rows = x.shape[0]
         plan = streaming_plan(rows, w_router.shape[0], w_router.shape[1], device=x.device) if rows <= SKINNY_AUTO_ROWS else None
         if plan is not None and plan[1] == 1:
             logits = gemm_skinny(x, w_router, torch.float32, block_shape=plan[0])
-        else:
+        elif rows > ROUTER_FUSED_MAX_ROWS:
             logits = gemm_rows_f32out(x, w_router)
-        if logits_out is not None:
+        if logits is not None and logits_out is not None:
             logits_out.copy_(logits)
     if logits is not None:
         _dev(logits)
