@@ -412,3 +412,21 @@ def test_one_matrix_per_head(dtype, n, heads, N, K):
         tol = 1e-5 if dtype == torch.float32 else 1e-2
         assert float((got[..., :N] - ref).abs().max()) <= tol * max(1.0, float(ref.abs().max())), f"gated={gated} form={form}"
         assert float(got[..., N:].abs().max()) == 0.0           # nothing is written between the heads
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_odd_width_and_a_cached_vector_above_256(tmp_path, dtype):
+    """A width that is no multiple of 4 (no kernel may take its 16-byte path), a cached vector of 288 elements
+    (beyond the matrix-core attention kernels: the float kernel runs in bfloat16 too), expert sizes that are no
+    multiples of 8 (float-FMA expert products in bfloat16), under a lightning layer with a key size of 6."""
+    small = dict(name="odd", seed=31, std=0.25, norm_std=0.2, config=config(50, 61, [
+        layer(latent(2, 16, 32, 8, 256, 24, window=40), moe(3, 2, 20, 12)),
+        layer(lightning(2, 6, 10, (0.8, 0.99)), moe(4, 1, 12)),
+    ]))
+    folder = make_folder(small, tmp_path)
+    cfg, w = plain_of(folder)
+    toks = tokens_of(cfg, 70, 8)
+    want = expected(cfg, w, toks, dtype)
+    core = make_core(folder, dtype, 16)
+    check_rows(dtype, run_cut(core, "whole", toks, [70]), want, "whole")
+    check_rows(dtype, run_cut(core, "cut", toks, [33, 2, 1, 17, 1, 1, 15]), want, "portions")
