@@ -163,7 +163,7 @@ def test_unused_tensors_are_named_and_tolerated_unless_strict(tmp_path, capsys):
     assert model.layers[0].mixer.w_qkv.shape == (4 * 16 + 2 * 2 * 16, 64)
     with pytest.raises(WeightsError, match="unexpected tensors \\(1\\): " + extra):
         load_model(folder, "float32", "cpu", strict=True)
-    # without strict the checker hands the names back and raises only for real problems
+    # without strict the shape check hands the names back and raises only for real problems
     arch, c, _ = resolve(TINY_A["config"])
     specs = DecoderModel(arch.build_spec(c)).tensor_specs()
     available = {k: (torch.bfloat16, tuple(v.shape)) for k, v in specs.items()}

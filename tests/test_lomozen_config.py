@@ -97,7 +97,7 @@ def test_bad_configurations_are_refused_with_the_key_named():
 
 
 def test_random_model_folder_round_trip(tmp_path):
-    """``write_random_model`` writes what the plain reader and the product's checker both accept."""
+    """``write_random_model`` writes what the plain reader and the loader's shape check both accept."""
     from jax_vllm_amd import write_random_model
     from jax_vllm_amd.weights.loader import check_against_specs
     from jax_vllm_amd.weights.safetensors_io import open_shards
