@@ -240,8 +240,10 @@ def test_greedy_generation_through_the_entry_point(folders, dtype):
     prompts = [tokens_of(cfg, n, 30 + n) for n in (3, 41, 18, 70)]
     llm = LLM(folders["C"], dtype=dtype, block_size=SMALL_C["page_size"], max_num_seqs=2, max_model_len=128,
               max_num_batched_tokens=24, num_blocks=9)
+    assert llm.prewarm() > 0.0            # records the decode steps of both batch sizes; leaves no trace in the state slots
     got = llm.generate(prompts, SamplingParams(max_new_tokens=12))
     assert [len(g) for g in got] == [12] * 4
+    assert llm.stats.graph_replays > 0
     for p, g in zip(prompts, got):
         seq = list(p)
         for i, t in enumerate(g):
