@@ -432,3 +432,23 @@ def test_odd_width_and_a_cached_vector_above_256(tmp_path, dtype):
     core = make_core(folder, dtype, 16)
     check_rows(dtype, run_cut(core, "whole", toks, [70]), want, "whole")
     check_rows(dtype, run_cut(core, "cut", toks, [33, 2, 1, 17, 1, 1, 15]), want, "portions")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_far_keys_without_a_window(tmp_path, dtype):
+    """Latent attention over every earlier key, scores sharp enough that one key among hundreds carries a row, as
+    often as not a far one: rows beyond position 200 change by much when the plain implementation is kept from
+    seeing keys more than 150 back.  300 tokens over 19 pages: whole, in portions that end at and around page
+    borders, and with the last 40 decoded one by one."""
+    mixer = dict(heads=2, dim=16, rot_dim=8, vdim=16, kv_rank=24, q_rank=24, scale=1.0)
+    small = dict(name="far", seed=23, std=0.3, norm_std=0.1, config=config(32, 50, [layer(latent(window=None, **mixer))]))
+    folder = make_folder(small, tmp_path)
+    cfg, w = plain_of(folder)
+    toks = tokens_of(cfg, 300, 12)
+    want = expected(cfg, w, toks, dtype)
+    plain = plain_logits(cfg, w, toks)
+    near = plain_logits(config(32, 50, [layer(latent(window=150, **mixer))]), w, toks)
+    assert np.median(np.abs(near[200:] - plain[200:]).max(axis=-1)) > 0.01 * np.abs(plain).max()
+    core = make_core(folder, dtype, 16, pages=20)
+    check_rows(dtype, run_cut(core, "whole", toks, [300]), want, "whole")
+    check_rows(dtype, run_cut(core, "portions", toks, [64, 63, 1, 17, 47, 2, 66] + [1] * 40), want, "portions and decoding")
