@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import torch
 
-from ..parts.spec import LayerMemory
+from ..parts.spec import LayerMemory, state_specs_of
 
 _STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
 
@@ -25,7 +25,7 @@ def group_keys_of(plan) -> list:
 
 
 def has_state(plan) -> bool:
-    return any(p.state is not None for p in plan)
+    return any(state_specs_of(p.state) for p in plan)
 
 
 def allocate_memories(plan, group_keys, num_pages, page_size: int, max_num_seqs: int, dtype, device) -> list:
@@ -56,9 +56,10 @@ def allocate_memories(plan, group_keys, num_pages, page_size: int, max_num_seqs:
                         f"run {p.run} cannot read run {p.cache_of}'s cache: it needs keys that the owner's "
                         f"window of {other.window} has already given back")
                 mem.pages, mem.group, mem.writes = owner.pages, owner.group, False
-        if p.state is not None:
+        for st in state_specs_of(p.state):
             # one row per slot and a spare one that belongs to no request
-            mem.state = torch.zeros((max_num_seqs + 1, *p.state.shape), dtype=_STATE_DTYPES[p.state.dtype], device=device)
+            mem.states[st.name] = torch.zeros((max_num_seqs + 1, *st.shape), dtype=_STATE_DTYPES[st.dtype], device=device)
+        mem.state = next(iter(mem.states.values()), None)
         memories.append(mem)
     return memories
 

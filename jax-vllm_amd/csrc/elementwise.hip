@@ -379,6 +379,29 @@ __global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bia
   *at = from_f32<T>(to_f32(*at) + bias[c]);
 }
 
+
+// y[r][c] = act(y[r][c] + bias[c]) in place, for a feed-forward whose activation stands alone (no gate).
+// act: 0 none, JV_ACT_SILU, JV_ACT_GELU_TANH, JV_ACT_GELU_ERF; computed in float.
+template <typename T>
+__global__ void bias_act_kernel(T* __restrict__ y, const float* __restrict__ bias, int n, int act) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n) return;
+  T* at = y + (long long)blockIdx.y * n + c;
+  *at = from_f32<T>(jv_act(act, to_f32(*at) + (bias ? bias[c] : 0.f)));
+}
+
+// out[i] = scale * ((rows ? rows[i] : 0) + parts[0][i] + parts[1][i] + ...) as float: one sublayer's
+// output (rows of the activation type and / or float partial results) weighed for a sum of several.
+template <typename T>
+__global__ void scaled_sum_kernel(float* __restrict__ out, const T* __restrict__ rows, const float* __restrict__ parts,
+                                  int n_parts, long long part_stride, long long n, float scale) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float v = rows ? to_f32(rows[i]) : 0.f;
+  for (int p = 0; p < n_parts; ++p) v += parts[p * part_stride + i];
+  out[i] = v * scale;
+}
+
 #define DEFINE_ELEMENTWISE(SUF, T)                                                                  \
   extern "C" int jv_embedding_##SUF(float* h, const void* table, const int* ids, int n_tokens,      \
                                     int hidden, int rows, void* stream) {                           \
@@ -470,6 +493,24 @@ __global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bia
     if (n_out <= 0) return 0;                                                                       \
     hipLaunchKernelGGL(cast_rows_kernel<T>, dim3(n_out), dim3(256), 0, (hipStream_t)stream,         \
                        (T*)out, x, rows, n);                                                        \
+    return JV_LAUNCH_CHECK();                                                                       \
+  }                                                                                                 \
+  extern "C" int jv_bias_act_##SUF(void* y, const float* bias, long long rows, int n, int act, void* stream) { \
+    if (rows <= 0 || n <= 0) return 0;                                                              \
+    if (act != 0 && !jv_plain_act_known(act)) return (int)hipErrorInvalidValue;                     \
+    for (long long r0 = 0; r0 < rows; r0 += 65535) { /* grid.y limit */                             \
+      const unsigned ny = (unsigned)(rows - r0 < 65535 ? rows - r0 : 65535);                        \
+      hipLaunchKernelGGL(bias_act_kernel<T>, dim3((n + 255) / 256, ny), dim3(256), 0,               \
+                         (hipStream_t)stream, (T*)y + r0 * n, bias, n, act);                        \
+    }                                                                                               \
+    return JV_LAUNCH_CHECK();                                                                       \
+  }                                                                                                 \
+  extern "C" int jv_scaled_sum_##SUF(float* out, const void* rows, const float* parts, int n_parts, \
+                                     long long part_stride, long long n, float scale, void* stream) { \
+    if (n <= 0) return 0;                                                                           \
+    if (!rows && n_parts <= 0) return (int)hipErrorInvalidValue;                                    \
+    hipLaunchKernelGGL(scaled_sum_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,       \
+                       (hipStream_t)stream, out, (const T*)rows, parts, n_parts, part_stride, n, scale); \
     return JV_LAUNCH_CHECK();                                                                       \
   }                                                                                                 \
   extern "C" int jv_add_bias_##SUF(void* y, const float* bias, long long rows, int n, void* stream) { \

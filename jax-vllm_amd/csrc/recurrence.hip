@@ -1,0 +1,331 @@
+// Recurrent mixers with a float matrix state per request and head, and what stands around them:
+//
+//   short_conv        a causal convolution over time per channel whose last taps - 1 inputs are state
+//   recurrence_gates  per (token, head): decay g = exp(-exp(A) softplus(raw + bias)) and a write strength
+//                     (the step size itself, or sigmoid of another column)
+//   heads_to_f32      heads of a projection as float, optionally rotated by position and scaled
+//   head_unit_norm    x / sqrt(sum(x^2) + eps) * scale per head, in place on the leading heads of every row
+//   recurrence_steps  S <- g S;  u = w (v - [delta] S^T k);  S <- S + k u^T;  o = S^T q (+ skip v)
+//   group_gated_norm  norm of float rows in equal groups, a gate before or behind it
+//
+// One recurrence serves retention (g constant per head, w = 1), the state-space form (k and q shared by a
+// group of heads, w = step size, skip) and the gated delta rule (delta = 1, w = beta).  Everything that
+// enters it is float.  The state of a request lives in a row of `state` [slots + 1][heads][dim][vdim]
+// between steps.  Columns of S never mix, so a block takes one (request, head, slice of columns) and a
+// thread keeps up to RC_ROWS rows of one column in registers.
+#include "common.h"
+
+#define RC_ROWS 32
+#define RC_MAX_LAGS 7        // a convolution has at most 8 taps
+
+__device__ __forceinline__ float rc_silu(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float rc_softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// ---------------------------------------------------------------- short causal convolution with state
+// out[t][c] = act( bias[c] + sum_j w[c][j] * in[t - (taps - 1) + j][c] ), in = proj[:, c_off + c] of the
+// request's tokens, continued to the left by the request's state rows [taps - 1][channels] (lag taps - 1
+// first).  grid (requests, channel blocks, segments of seg_len tokens); the thread of segment 0 also
+// writes the state the step leaves (it is the only one that reads the old one).
+template <typename T>
+__global__ void __launch_bounds__(256)
+short_conv_kernel(float* __restrict__ out, long long ldo, const T* __restrict__ proj, long long ld, int c_off,
+                  int channels, int taps, const float* __restrict__ w, const float* __restrict__ bias,
+                  float* __restrict__ state, const int* __restrict__ slot_ids, const int* __restrict__ cu_seqlens,
+                  int act, int seg_len) {
+  const int r = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= channels) return;
+  const int t0 = cu_seqlens[r], n = cu_seqlens[r + 1] - t0;
+  const int s0 = blockIdx.z * seg_len;
+  if (s0 >= n) return;
+  const int lags = taps - 1;
+  float* st = state + (long long)slot_ids[r] * lags * channels + c;
+  const T* in = proj + (long long)t0 * ld + c_off + c;
+  // slot p of the window holds the input of lag RC_MAX_LAGS - p; lags the filter does not have weigh nothing
+  float win[RC_MAX_LAGS], wl[RC_MAX_LAGS];
+#pragma unroll
+  for (int p = 0; p < RC_MAX_LAGS; ++p) {
+    const int lag = RC_MAX_LAGS - p;
+    float x = 0.f, f = 0.f;
+    if (lag <= lags) {
+      f = w[(long long)c * taps + lags - lag];
+      const int i = s0 - lag;
+      x = i >= 0 ? to_f32(in[(long long)i * ld]) : st[(long long)(lags + i) * channels];
+    }
+    win[p] = x;
+    wl[p] = f;
+  }
+  const float w0 = w[(long long)c * taps + lags], b = bias ? bias[c] : 0.f;
+  const int s1 = min(n, s0 + seg_len);
+  for (int i = s0; i < s1; ++i) {
+    const float x = to_f32(in[(long long)i * ld]);
+    float acc = b;
+#pragma unroll
+    for (int p = 0; p < RC_MAX_LAGS; ++p) acc = fmaf(wl[p], win[p], acc);
+    acc = fmaf(w0, x, acc);
+    out[(long long)(t0 + i) * ldo + c] = act ? rc_silu(acc) : acc;
+#pragma unroll
+    for (int p = 0; p + 1 < RC_MAX_LAGS; ++p) win[p] = win[p + 1];
+    win[RC_MAX_LAGS - 1] = x;
+  }
+  if (blockIdx.z == 0) {
+    // the last `lags` inputs of the request: rows of this step, or, for a short step, old state rows moved up
+    // (row j takes row j + n: read before any row above j is written)
+    for (int j = 0; j < lags; ++j) {
+      const int i = n - lags + j;
+      st[(long long)j * channels] = i >= 0 ? to_f32(in[(long long)i * ld]) : st[(long long)(j + n) * channels];
+    }
+  }
+}
+
+// ---------------------------------------------------------------- decays and write strengths
+// mode 0: dt = softplus(raw + bias);  g = exp(-exp(A) dt);  w = dt
+// mode 1: g as above from the column at dt_off;  w = sigmoid(column at w_off)
+template <typename T>
+__global__ void __launch_bounds__(256)
+recurrence_gates_kernel(float* __restrict__ g, float* __restrict__ wgt, const T* __restrict__ proj, long long ld,
+                        int dt_off, int w_off, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                        int n, int heads, int mode) {
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (long long)n * heads) return;
+  const int t = (int)(e / heads), h = (int)(e % heads);
+  const float dt = rc_softplus(to_f32(proj[(long long)t * ld + dt_off + h]) + dt_bias[h]);
+  g[e] = expf(-expf(a_log[h]) * dt);
+  wgt[e] = mode == 0 ? dt : 1.f / (1.f + expf(-to_f32(proj[(long long)t * ld + w_off + h])));
+}
+
+// ---------------------------------------------------------------- heads as float, rotated and scaled
+// out[t][h][i] of `width` = heads * d columns of proj from `off`; the first rot_dims elements of a head turn
+// by the token's angles (cos_sin [n][rot_dims]: cosines, then sines; element i pairs with i + rot_dims / 2).
+template <typename T>
+__global__ void __launch_bounds__(256)
+heads_to_f32_kernel(float* __restrict__ out, const T* __restrict__ proj, long long ld, int off, int n, int heads,
+                    int d, int rot_dims, const float* __restrict__ cos_sin, float scale) {
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+  const int width = heads * d;
+  if (e >= (long long)n * width) return;
+  const int t = (int)(e / width), c = (int)(e % width), i = c % d;
+  const T* row = proj + (long long)t * ld + off;
+  float x = to_f32(row[c]);
+  if (i < rot_dims) {
+    const int half = rot_dims / 2, j = i < half ? i : i - half;
+    const float cs = cos_sin[(long long)t * rot_dims + j], sn = cos_sin[(long long)t * rot_dims + half + j];
+    const float other = to_f32(row[i < half ? c + half : c - half]);
+    x = i < half ? x * cs - other * sn : x * cs + other * sn;
+  }
+  out[e] = x * scale;
+}
+
+// x [n][ld] float, in place on the first `heads` runs of d columns of every row: x / sqrt(sum(x^2) + eps) * scale,
+// scale = scale_a for the first `heads_a` heads of a row and scale_b for the others; one wave a head
+__global__ void __launch_bounds__(256)
+head_unit_norm_kernel(float* __restrict__ x, long long ld, long long n, int heads, int d, float eps, int heads_a,
+                      float scale_a, float scale_b) {
+  const long long r = (long long)blockIdx.x * 4 + threadIdx.x / JV_WAVE;
+  if (r >= n * heads) return;
+  const int lane = threadIdx.x % JV_WAVE;
+  const int hd = (int)(r % heads);
+  float* p = x + (r / heads) * ld + (long long)hd * d;
+  float ss = 0.f;
+  for (int i = lane; i < d; i += JV_WAVE) ss = fmaf(p[i], p[i], ss);
+  ss = wave_sum(ss);
+  const float inv = (hd < heads_a ? scale_a : scale_b) / sqrtf(ss + eps);
+  for (int i = lane; i < d; i += JV_WAVE) p[i] *= inv;
+}
+
+// ---------------------------------------------------------------- the recurrence, token by token
+// grid (requests, heads, column slices); block 256 = parts x cols threads, cols a power of two.
+// q, k: [n][qk_heads][dim] (row strides ldq, ldk), head h reads qk head h / (heads / qk_heads);
+// v: [n][heads][vdim]; g: [n][heads] (g_stride = heads) or [heads] (g_stride = 0); wgt [n][heads] or null (1);
+// skip [heads] or null: out += skip[h] * v.
+__global__ void __launch_bounds__(256)
+recurrence_steps_kernel(float* __restrict__ out, const float* __restrict__ q, long long ldq,
+                        const float* __restrict__ k, long long ldk, const float* __restrict__ v, long long ldv,
+                        const float* __restrict__ g, int g_stride, const float* __restrict__ wgt,
+                        const float* __restrict__ skip, float* __restrict__ state, const int* __restrict__ slot_ids,
+                        const int* __restrict__ cu_seqlens, int heads, int qk_heads, int dim, int vdim, int cols,
+                        int delta) {
+  extern __shared__ float lds[];          // 2 x (q[dim] | k[dim] | v[cols]) | two arrays of partial sums [parts][cols]
+  const int r = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * cols;
+  const int parts = blockDim.x / cols;
+  const int col = threadIdx.x % cols, part = threadIdx.x / cols;
+  const int t0 = cu_seqlens[r], t1 = cu_seqlens[r + 1];
+  if (t1 <= t0) return;
+  const int stage = 2 * dim + cols;
+  float* red_a = lds + 2 * stage;
+  float* red_b = red_a + parts * cols;
+  const int hk = h / (heads / qk_heads);
+  const bool live = c0 + col < vdim;
+  const float sk = skip ? skip[h] : 0.f;
+  float* S = state + (((long long)slot_ids[r] * heads + h) * dim) * vdim + c0 + col;
+  float s[RC_ROWS];
+#pragma unroll
+  for (int i = 0; i < RC_ROWS; ++i) {
+    const int d = part + i * parts;
+    s[i] = (live && d < dim) ? S[(long long)d * vdim] : 0.f;
+  }
+  for (int t = t0; t < t1; ++t) {
+    float* buf = lds + ((t - t0) & 1) * stage;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+      buf[d] = q[(long long)t * ldq + hk * dim + d];
+      buf[dim + d] = k[(long long)t * ldk + hk * dim + d];
+    }
+    if (threadIdx.x < cols)
+      buf[2 * dim + threadIdx.x] = (c0 + threadIdx.x < vdim) ? v[(long long)t * ldv + h * vdim + c0 + threadIdx.x] : 0.f;
+    const float gt = g[(long long)t * g_stride + h];
+    const float wt = wgt ? wgt[(long long)t * heads + h] : 1.f;
+    __syncthreads();
+    const float vv = buf[2 * dim + col];
+    float u = wt * vv;
+    if (delta) {
+      float pred = 0.f;
+#pragma unroll
+      for (int i = 0; i < RC_ROWS; ++i) {
+        const int d = part + i * parts;
+        if (d < dim) {
+          s[i] *= gt;
+          pred = fmaf(s[i], buf[dim + d], pred);
+        }
+      }
+      red_a[part * cols + col] = pred;
+      __syncthreads();
+      pred = 0.f;
+      for (int p = 0; p < parts; ++p) pred += red_a[p * cols + col];
+      u = wt * (vv - pred);
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < RC_ROWS; ++i) {
+      const int d = part + i * parts;
+      if (d < dim) {
+        s[i] = delta ? fmaf(buf[dim + d], u, s[i]) : fmaf(gt, s[i], buf[dim + d] * u);
+        acc = fmaf(s[i], buf[d], acc);
+      }
+    }
+    red_b[part * cols + col] = acc;
+    __syncthreads();
+    if (part == 0 && live) {
+      float o = 0.f;
+      for (int p = 0; p < parts; ++p) o += red_b[p * cols + col];
+      out[(long long)t * heads * vdim + h * vdim + c0 + col] = fmaf(sk, vv, o);
+    }
+    // the next token fills the other stage; red_a and red_b are rewritten only behind the barrier after that fill
+  }
+#pragma unroll
+  for (int i = 0; i < RC_ROWS; ++i) {
+    const int d = part + i * parts;
+    if (live && d < dim) S[(long long)d * vdim] = s[i];
+  }
+}
+
+// ---------------------------------------------------------------- norm in groups with a gate
+//   a = gate_first ? o * act(gate) : o;   y = a * rsqrt(mean_group(a^2) + eps) * w[c % w_period];
+//   out = T( (gate_first ? y : y * act(gate)) * out_scale );   act: 1 silu, 2 sigmoid;  w null: no weight
+// grid (rows, ceil(groups / 4)); one wave a group.
+template <typename T>
+__global__ void __launch_bounds__(256)
+group_gated_norm_kernel(T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ gate,
+                        long long g_stride, const float* __restrict__ w, int w_period, int width, int group,
+                        float eps, int gate_act, int gate_first, float out_scale) {
+  const long long t = blockIdx.x;
+  const int grp = blockIdx.y * 4 + threadIdx.x / JV_WAVE, lane = threadIdx.x % JV_WAVE;
+  if (grp * group >= width) return;
+  const float* x = o + t * width + grp * group;
+  const T* gp = gate + t * g_stride + grp * group;
+  float ss = 0.f;
+  for (int i = lane; i < group; i += JV_WAVE) {
+    float a = x[i];
+    if (gate_first) {
+      const float z = to_f32(gp[i]);
+      a *= gate_act == 1 ? rc_silu(z) : 1.f / (1.f + expf(-z));
+    }
+    ss = fmaf(a, a, ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = rsqrtf(ss / (float)group + eps) * out_scale;
+  for (int i = lane; i < group; i += JV_WAVE) {
+    const float z = to_f32(gp[i]);
+    const float ga = gate_act == 1 ? rc_silu(z) : 1.f / (1.f + expf(-z));
+    const float wv = w ? w[(grp * group + i) % w_period] : 1.f;
+    out[t * width + grp * group + i] = from_f32<T>(x[i] * ga * inv * wv);
+  }
+}
+
+extern "C" int jv_recurrence_max_dim() { return RC_ROWS * 256; }
+extern "C" int jv_short_conv_max_taps() { return RC_MAX_LAGS + 1; }
+
+extern "C" int jv_head_unit_norm(float* x, long long ld, long long n, int heads, int d, float eps, int heads_a,
+                                 float scale_a, float scale_b, void* stream) {
+  if (n <= 0 || heads <= 0 || d <= 0) return 0;
+  if ((long long)heads * d > ld) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(head_unit_norm_kernel, dim3((unsigned)((n * heads + 3) / 4)), dim3(256), 0, (hipStream_t)stream, x,
+                     ld, n, heads, d, eps, heads_a, scale_a, scale_b);
+  return JV_LAUNCH_CHECK();
+}
+
+extern "C" int jv_recurrence_steps(float* out, const float* q, long long ldq, const float* k, long long ldk,
+                                   const float* v, long long ldv, const float* g, int g_stride, const float* wgt,
+                                   const float* skip, float* state, const int* slot_ids, const int* cu_seqlens,
+                                   int n_requests, int heads, int qk_heads, int dim, int vdim, int delta,
+                                   void* stream) {
+  if (n_requests <= 0 || heads <= 0) return 0;
+  if (dim <= 0 || vdim <= 0 || heads > 65535 || qk_heads <= 0 || heads % qk_heads) return (int)hipErrorInvalidValue;
+  int cols = 64;                       /* the widest slice that keeps a thread's rows in registers */
+  while (cols > 1 && (cols / 2 >= vdim || (long long)dim * cols > 256LL * RC_ROWS)) cols /= 2;
+  if ((long long)dim * cols > 256LL * RC_ROWS) return (int)hipErrorInvalidValue;
+  const int parts = 256 / cols;
+  const size_t shmem = (2 * (2 * dim + cols) + 2 * parts * cols) * sizeof(float);
+  hipLaunchKernelGGL(recurrence_steps_kernel, dim3(n_requests, heads, (vdim + cols - 1) / cols), dim3(256), shmem,
+                     (hipStream_t)stream, out, q, ldq, k, ldk, v, ldv, g, g_stride, wgt, skip, state, slot_ids,
+                     cu_seqlens, heads, qk_heads, dim, vdim, cols, delta);
+  return JV_LAUNCH_CHECK();
+}
+
+#define DEFINE_RECURRENCE(SUF, T)                                                                              \
+  extern "C" int jv_short_conv_##SUF(float* out, long long ldo, const void* proj, long long ld, int c_off,     \
+                                     int channels, int taps, const float* w, const float* bias, float* state,  \
+                                     const int* slot_ids, const int* cu_seqlens, int n_requests,               \
+                                     int max_q_len, int act, void* stream) {                                   \
+    if (n_requests <= 0 || channels <= 0 || max_q_len <= 0) return 0;                                          \
+    if (taps < 1 || taps > RC_MAX_LAGS + 1) return (int)hipErrorInvalidValue;                                  \
+    const int seg_len = 64;                                                                                    \
+    hipLaunchKernelGGL(short_conv_kernel<T>, dim3(n_requests, (channels + 255) / 256,                          \
+                                                  (max_q_len + seg_len - 1) / seg_len),                        \
+                       dim3(256), 0, (hipStream_t)stream, out, ldo, (const T*)proj, ld, c_off, channels, taps, \
+                       w, bias, state, slot_ids, cu_seqlens, act, seg_len);                                    \
+    return JV_LAUNCH_CHECK();                                                                                  \
+  }                                                                                                            \
+  extern "C" int jv_recurrence_gates_##SUF(float* g, float* wgt, const void* proj, long long ld, int dt_off,   \
+                                           int w_off, const float* dt_bias, const float* a_log, int n,         \
+                                           int heads, int mode, void* stream) {                                \
+    if (n <= 0 || heads <= 0) return 0;                                                                        \
+    hipLaunchKernelGGL(recurrence_gates_kernel<T>, dim3((unsigned)(((long long)n * heads + 255) / 256)),       \
+                       dim3(256), 0, (hipStream_t)stream, g, wgt, (const T*)proj, ld, dt_off, w_off, dt_bias,  \
+                       a_log, n, heads, mode);                                                                 \
+    return JV_LAUNCH_CHECK();                                                                                  \
+  }                                                                                                            \
+  extern "C" int jv_heads_to_f32_##SUF(float* out, const void* proj, long long ld, int off, int n, int heads,  \
+                                       int d, int rot_dims, const float* cos_sin, float scale, void* stream) { \
+    if (n <= 0 || heads <= 0 || d <= 0) return 0;                                                              \
+    if (rot_dims < 0 || rot_dims > d || rot_dims % 2 || (rot_dims && !cos_sin)) return (int)hipErrorInvalidValue; \
+    hipLaunchKernelGGL(heads_to_f32_kernel<T>, dim3((unsigned)(((long long)n * heads * d + 255) / 256)),       \
+                       dim3(256), 0, (hipStream_t)stream, out, (const T*)proj, ld, off, n, heads, d, rot_dims, \
+                       cos_sin, scale);                                                                        \
+    return JV_LAUNCH_CHECK();                                                                                  \
+  }                                                                                                            \
+  extern "C" int jv_group_gated_norm_##SUF(void* out, const float* o, const void* gate, long long g_stride,    \
+                                           const float* w, int w_period, int n, int width, int group,          \
+                                           float eps, int gate_act, int gate_first, float out_scale,           \
+                                           void* stream) {                                                     \
+    if (n <= 0 || width <= 0) return 0;                                                                        \
+    if (group <= 0 || width % group || (w && w_period <= 0) || (gate_act != 1 && gate_act != 2))               \
+      return (int)hipErrorInvalidValue;                                                                        \
+    const int groups = width / group;                                                                          \
+    if (groups > 4 * 65535) return (int)hipErrorInvalidValue;                                                  \
+    hipLaunchKernelGGL(group_gated_norm_kernel<T>, dim3(n, (groups + 3) / 4), dim3(256), 0,                    \
+                       (hipStream_t)stream, (T*)out, o, (const T*)gate, g_stride, w, w_period, width, group,   \
+                       eps, gate_act, gate_first, out_scale);                                                  \
+    return JV_LAUNCH_CHECK();                                                                                  \
+  }
+
+DEFINE_RECURRENCE(bf16, bf16_t)
+DEFINE_RECURRENCE(f32, float)

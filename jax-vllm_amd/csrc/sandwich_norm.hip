@@ -8,7 +8,7 @@
 //   v   = (y ? y[r] : 0) + parts[0][r] + parts[1][r] + ...       (the sublayer's output; parts added in order)
 //   x   = h[r] + v * rsqrt(mean(v^2) + eps) * wb                 (float)
 //   if (!rows) h[r] = x
-//   if (out)   out[i] = T( x * rsqrt(mean(x^2) + eps_out) * w )
+//   if (out)   out[i] = T( x * rsqrt(mean(x^2) + eps_out) * w ),   or T(x) where w is null
 // One block per output row; the row is kept in LDS between the passes (hidden floats).
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -38,9 +38,13 @@ postnorm_add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ y, cons
     ss2 += x * x;
   }
   if (!out) return;
+  T* o = out + i * hidden;
+  if (!w) {          // the reader takes the stream itself: no norm, the row in the activation type
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) o[c] = from_f32<T>(row[c]);
+    return;
+  }
   ss2 = block_sum(ss2, red);
   const float inv = rsqrtf(ss2 / (float)hidden + eps_out);
-  T* o = out + i * hidden;
   for (int c = threadIdx.x; c < hidden; c += blockDim.x) o[c] = from_f32<T>(row[c] * inv * w[c]);
 }
 
@@ -126,6 +130,14 @@ postnorm_add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ y, 
     }
   }
   if (!out) return;
+  if (!w) {          // the reader takes the stream itself: no norm, the row in the activation type
+#pragma unroll
+    for (int q = 0; q < SN_V; ++q) {
+      const int c = (threadIdx.x + q * 256) * 4;
+      if (c < hidden) sn_store4<T>(out + i * hidden + c, x[q]);
+    }
+    return;
+  }
   ss2 = block_sum(ss2, red);
   const float inv = rsqrtf(ss2 / (float)hidden + eps_out);
 #pragma unroll

@@ -270,8 +270,8 @@ class EngineCore:
             # rows that pad the step write the spare state row: it starts from zero in every step, so
             # that a mixer which keeps adding to its state never runs it up to infinity there
             for m in self.memories:
-                if m.state is not None:
-                    m.state[self._spare_slot].zero_()
+                for st in m.states.values():
+                    st[self._spare_slot].zero_()
         g.dev.copy_(g.host_tensor, non_blocking=True)
         if g.copied is None:
             g.copied = torch.cuda.Event()
@@ -298,11 +298,11 @@ class EngineCore:
 
     def _zero_new_state(self) -> None:
         slots = self.cache.take_new_slots()
-        if slots and any(m.state is not None for m in self.memories):
+        if slots and any(m.states for m in self.memories):
             idx = torch.tensor(slots, dtype=torch.long, device=self.device)
             for m in self.memories:
-                if m.state is not None:
-                    m.state.index_fill_(0, idx, 0)
+                for st in m.states.values():
+                    st.index_fill_(0, idx, 0)
 
     def _build(self, entries):
         """All per-token and per-request integers of the step, packed on the host into one

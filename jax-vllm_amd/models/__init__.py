@@ -1,2 +1,3 @@
 from . import qwen3  # noqa: F401  (registers Qwen3ForCausalLM)
 from . import lomozen  # noqa: F401  (registers Lomozen)
+from . import dumazen  # noqa: F401  (registers Dumazen)

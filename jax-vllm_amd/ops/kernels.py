@@ -199,6 +199,39 @@ def add_bias(y: torch.Tensor, bias: torch.Tensor) -> None:
     _check(fn(_ptr(rows), _ptr(bias), c_longlong(rows.shape[0]), c_int(rows.shape[1]), _stream()), "add_bias")
 
 
+PLAIN_ACTIVATIONS = {None: 0, "silu": 1, "gelu_tanh": 2, "gelu": 3}     # ids of act in y = act(x + bias); "gelu" is the erf form
+
+
+def bias_act(y: torch.Tensor, bias, activation) -> None:
+    """y[r, c] = act(y[r, c] + bias[c]) in place for contiguous rows; ``bias`` float32 or None, ``activation`` one of
+    ``PLAIN_ACTIVATIONS`` (None: the bias alone); computed in float."""
+    _dev(y, bias)
+    _need(y.dim() == 2, "y must be rows")
+    _need(activation in PLAIN_ACTIVATIONS, f"no kernel for the activation {activation!r}: there are {sorted(map(str, PLAIN_ACTIVATIONS))}")
+    if bias is not None:
+        _f32(bias, "bias", y.shape[1])
+    fn = getattr(library.core(), f"jv_bias_act_{_suffix(y.dtype)}")
+    _check(fn(_ptr(y), _ptr(bias), c_longlong(y.shape[0]), c_int(y.shape[1]), c_int(PLAIN_ACTIVATIONS[activation]), _stream()),
+           "bias_act")
+
+
+def scaled_sum(out: torch.Tensor, y, scale: float) -> None:
+    """out = scale * y as float, where ``y`` is what a sublayer returned: rows of the activation type, a float stack
+    [P, rows, width] of partial results (added in order), or a pair (rows or None, stack or None)."""
+    rows, parts = split_sublayer_output(y)
+    _dev(out, rows, parts)
+    _f32(out, "out")
+    _need(rows is not None or parts is not None, "nothing to add")
+    if rows is not None:
+        _need(rows.shape == out.shape, "rows must match out's shape")
+    if parts is not None:
+        _need(parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[1:] == out.shape, "parts must be float32 [P, *out.shape]")
+    kind = rows.dtype if rows is not None else torch.float32
+    fn = getattr(library.core(), f"jv_scaled_sum_{_suffix(kind)}")
+    _check(fn(_ptr(out), _ptr(rows), _ptr(parts), c_int(0 if parts is None else parts.shape[0]),
+              c_longlong(0 if parts is None else parts.stride(0)), c_longlong(out.numel()), c_float(scale), _stream()), "scaled_sum")
+
+
 # --------------------------------------------------------------------------- activation
 GATE_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2}      # the kernels' ids of act in y = act(gate) * up
 
@@ -299,6 +332,46 @@ def qk_norm_rope_write(qkv, slot_mapping, q_weight, k_weight, eps, cos_sin, rota
            c_int(nq), c_int(nkv), c_int(head_dim), _stream()),
         "qk_norm_rope_write",
     )
+
+
+def padded_head_dim(dk: int, dv: int) -> int:
+    """The one head size under which keys of ``dk`` and values of ``dv`` elements are cached (zeros behind them):
+    the next multiple of 16, which the matrix-core attention kernels are built for."""
+    return -(-max(int(dk), int(dv)) // 16) * 16
+
+
+def attn_prepare_wide(qkv, bias, q_weight, k_weight, eps: float, cos_sin, rot_dims: int, slot_mapping, k_pages, v_pages,
+                      page_size: int, nq: int, nkv: int, dk: int, dv: int, dp: int, v_scale: float = 1.0) -> torch.Tensor:
+    """Attention input whose key and value sizes differ or whose q/k norm spans the whole projection.  ``qkv`` rows
+    are [q: nq * dk | k: nkv * dk | v: nkv * dv]; ``bias`` (float32, that width) is added first; with
+    ``q_weight`` [nq * dk] and ``k_weight`` [nkv * dk] q and k are RMS-normed over all their columns at once; the
+    first ``rot_dims`` elements of every q and k head turn by ``cos_sin`` (``rope_table``); v is multiplied by
+    ``v_scale``.  Returns q as [n, nq * dp] with every head padded with zeros to ``dp``; keys go to
+    [pages, nkv, page_size, dp], values to [pages, nkv, dp, page_size] (their pad is never written)."""
+    _dev(qkv, bias, q_weight, k_weight, cos_sin, slot_mapping, k_pages, v_pages)
+    n, ld = qkv.shape
+    width = (nq + nkv) * dk + nkv * dv
+    _need(ld == width, "qkv must be [tokens, nq * dk + nkv * dk + nkv * dv]")
+    _need(dp >= max(dk, dv), "the padded head size must hold keys and values")
+    if bias is not None:
+        _f32(bias, "bias", width)
+    _need((q_weight is None) == (k_weight is None), "q and k are normed together or not at all")
+    if q_weight is not None:
+        _f32(q_weight, "q_weight", nq * dk)
+        _f32(k_weight, "k_weight", nkv * dk)
+    _need(rot_dims % 2 == 0 and 0 <= rot_dims <= dk, "the rotated size must be even and at most the key size")
+    if rot_dims:
+        _f32(cos_sin, "cos_sin", n * rot_dims)
+    if k_pages is not None:
+        _i32(slot_mapping, "slot_mapping", n)
+        _check_pages(k_pages, v_pages, qkv.dtype, nkv, page_size, dp)
+    q = torch.empty((n, nq * dp), dtype=qkv.dtype, device=qkv.device)
+    fn = getattr(library.core(), f"jv_attn_prepare_wide_{_suffix(qkv.dtype)}")
+    _check(fn(_ptr(q), _ptr(qkv), c_longlong(ld), _ptr(bias), _ptr(q_weight), _ptr(k_weight), c_float(eps),
+              _ptr(cos_sin if rot_dims else None), c_int(rot_dims), _ptr(slot_mapping if k_pages is not None else None),
+              _ptr(k_pages), _ptr(v_pages), c_int(page_size), c_int(n), c_int(nq), c_int(nkv), c_int(dk), c_int(dv),
+              c_int(dp), c_float(v_scale), _stream()), "attn_prepare_wide")
+    return q
 
 
 # --------------------------------------------------------------------------- attention
@@ -811,7 +884,8 @@ def split_sublayer_output(out):
 def postnorm_add_rmsnorm(h, y, parts, post_weight, eps: float, weight=None, out=None, rows=None,
                          out_eps: float | None = None) -> None:
     """h += norm(y + parts[0] + parts[1] + ...; post_weight) in the float residual stream, then, with
-    ``out``, out = norm(h; weight) (with ``out_eps``, default ``eps``) in the activation type.  With ``rows`` (int32 indices) only those
+    ``out``, out = norm(h; weight) (with ``out_eps``, default ``eps``) in the activation type, or h itself in that type where
+    ``weight`` is None (a reader that takes the stream as it is).  With ``rows`` (int32 indices) only those
     rows are computed and h is left alone.  y is [rows of h, hidden] in the activation type or None,
     parts a float32 stack [P, rows of h, hidden] or None (any P)."""
     _dev(h, y, parts, post_weight, weight, out, rows)
@@ -826,7 +900,8 @@ def postnorm_add_rmsnorm(h, y, parts, post_weight, eps: float, weight=None, out=
         _need(parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[1:] == h.shape,
               "parts must be float32 [P, *h.shape]")
     if out is not None:
-        _f32(weight, "weight", hidden)
+        if weight is not None:       # None: out is the stream itself in the activation type, not normed
+            _f32(weight, "weight", hidden)
         n_out = out.shape[0]
         _need(out.shape[-1] == hidden, "out width differs from h")
         _need(y is None or y.dtype == out.dtype, "y and out must have one type")
@@ -998,6 +1073,154 @@ def lightning_attention(proj, q_off: int, k_off: int, v_off: int, state, slot_id
     _check(fn(_ptr(out), _ptr(proj), c_longlong(ld), c_int(q_off), c_int(k_off), c_int(v_off), _ptr(state),
               _ptr(slot_ids), _ptr(cu_seqlens), _ptr(decay), c_int(r), c_int(heads), c_int(dim), c_int(vdim),
               c_int(chunks), _ptr(work), _ptr(first), _ptr(scratch), _stream()), "lightning_attention")
+    return out
+
+
+# --------------------------------------------------------------------------- recurrences with a matrix state
+def short_conv_max_taps() -> int:
+    return library.core().jv_short_conv_max_taps()
+
+
+def recurrence_max_dim() -> int:
+    return library.core().jv_recurrence_max_dim()
+
+
+def short_conv(proj, c_off: int, channels: int, weight, bias, state, slot_ids, cu_seqlens, max_q_len: int,
+               activation: bool = True) -> torch.Tensor:
+    """Float [n, channels]: a causal convolution over time per channel of the columns ``proj[:, c_off : c_off +
+    channels]``, request by request; ``weight`` [channels, taps] (the last column weighs the current token), ``bias``
+    [channels] or None, then silu if ``activation``.  ``state`` [slots + 1, taps - 1, channels] float holds every
+    request's last taps - 1 inputs before the step and after it (zeros stand before a sequence's first token)."""
+    _dev(proj, weight, bias, state, slot_ids, cu_seqlens)
+    n, ld = proj.shape
+    r = slot_ids.numel()
+    _need(weight.dim() == 2 and weight.shape[0] == channels, "weight must be [channels, taps]")
+    taps = weight.shape[1]
+    _f32(weight, "weight")
+    _need(1 <= taps <= short_conv_max_taps(), f"a convolution of {taps} taps: the kernel takes up to {short_conv_max_taps()}")
+    if bias is not None:
+        _f32(bias, "bias", channels)
+    _f32(state, "state")
+    _need(state.dim() == 3 and tuple(state.shape[1:]) == (taps - 1, channels), "state must be [slots, taps - 1, channels]")
+    _need(0 <= c_off and c_off + channels <= ld, "proj rows are too short")
+    _i32(slot_ids, "slot_ids")
+    _i32(cu_seqlens, "cu_seqlens", r + 1)
+    out = torch.empty((n, channels), dtype=torch.float32, device=proj.device)
+    fn = getattr(library.core(), f"jv_short_conv_{_suffix(proj.dtype)}")
+    _check(fn(_ptr(out), c_longlong(channels), _ptr(proj), c_longlong(ld), c_int(c_off), c_int(channels), c_int(taps),
+              _ptr(weight), _ptr(bias), _ptr(state), _ptr(slot_ids), _ptr(cu_seqlens), c_int(r), c_int(max(1, int(max_q_len))),
+              c_int(1 if activation else 0), _stream()), "short_conv")
+    return out
+
+
+def recurrence_gates(proj, dt_off: int, dt_bias, a_log, heads: int, beta_off: "int | None" = None):
+    """(decay, write strength), float [n, heads] each, from columns of ``proj``: dt = softplus(proj[:, dt_off + h] +
+    dt_bias[h]) without a clamp, decay = exp(-exp(a_log[h]) * dt); the write strength is dt itself, or with
+    ``beta_off`` sigmoid(proj[:, beta_off + h])."""
+    _dev(proj, dt_bias, a_log)
+    n, ld = proj.shape
+    _f32(dt_bias, "dt_bias", heads)
+    _f32(a_log, "a_log", heads)
+    _need(0 <= dt_off and dt_off + heads <= ld and (beta_off is None or 0 <= beta_off and beta_off + heads <= ld), "proj rows are too short")
+    g = torch.empty((n, heads), dtype=torch.float32, device=proj.device)
+    w = torch.empty((n, heads), dtype=torch.float32, device=proj.device)
+    fn = getattr(library.core(), f"jv_recurrence_gates_{_suffix(proj.dtype)}")
+    _check(fn(_ptr(g), _ptr(w), _ptr(proj), c_longlong(ld), c_int(dt_off), c_int(0 if beta_off is None else beta_off),
+              _ptr(dt_bias), _ptr(a_log), c_int(n), c_int(heads), c_int(0 if beta_off is None else 1), _stream()), "recurrence_gates")
+    return g, w
+
+
+def heads_to_f32(proj, off: int, heads: int, d: int, rot_dims: int = 0, cos_sin=None, scale: float = 1.0) -> torch.Tensor:
+    """Float [n, heads * d] of the columns ``proj[:, off : off + heads * d]``; the first ``rot_dims`` elements of every
+    head turn by the token's angles (``rope_table``; element i pairs with i + rot_dims / 2); all times ``scale``."""
+    _dev(proj, cos_sin)
+    n, ld = proj.shape
+    _need(0 <= off and off + heads * d <= ld, "proj rows are too short")
+    _need(rot_dims % 2 == 0 and 0 <= rot_dims <= d, "the rotated size must be even and at most the head size")
+    if rot_dims:
+        _f32(cos_sin, "cos_sin", n * rot_dims)
+    out = torch.empty((n, heads * d), dtype=torch.float32, device=proj.device)
+    fn = getattr(library.core(), f"jv_heads_to_f32_{_suffix(proj.dtype)}")
+    _check(fn(_ptr(out), _ptr(proj), c_longlong(ld), c_int(off), c_int(n), c_int(heads), c_int(d), c_int(rot_dims),
+              _ptr(cos_sin if rot_dims else None), c_float(scale), _stream()), "heads_to_f32")
+    return out
+
+
+def head_unit_norm(x: torch.Tensor, heads: int, d: int, eps: float, scale: float = 1.0, first_heads: int = 0,
+                   first_scale: float = 1.0) -> None:
+    """In place on float rows [n, width]: each of the first ``heads`` runs of ``d`` columns of every row becomes
+    x / sqrt(sum(x^2) + eps) * scale; the first ``first_heads`` of them take ``first_scale`` instead."""
+    _dev(x)
+    _f32(x, "x")
+    _need(x.dim() == 2 and d > 0 and heads * d <= x.shape[1], "the heads do not fit the rows")
+    _check(library.core().jv_head_unit_norm(_ptr(x), c_longlong(x.shape[1]), c_longlong(x.shape[0]), c_int(heads), c_int(d),
+                                            c_float(eps), c_int(first_heads), c_float(first_scale), c_float(scale), _stream()),
+           "head_unit_norm")
+
+
+def recurrence_steps(q, k, v, decay, state, slot_ids, cu_seqlens, heads: int, qk_heads: int, dim: int, vdim: int,
+                     write=None, skip=None, delta: bool = False) -> torch.Tensor:
+    """Float [n, heads * vdim], token by token per request and head, S [dim, vdim] float in the request's state row:
+
+        S <- g S;   u = w (v - S^T k) if ``delta`` else w v;   S <- S + k u^T;   o = S^T q + skip[h] v
+
+    ``q``, ``k``: float views [n, qk_heads * dim] (unit column stride; head h reads q/k head h // (heads // qk_heads)),
+    ``v`` a float view [n, heads * vdim]; ``decay`` g: float [n, heads] or [heads] (constant per head); ``write`` w:
+    float [n, heads] or None (1); ``skip``: float [heads] or None."""
+    _dev(decay, write, skip, state, slot_ids, cu_seqlens)
+    n = v.shape[0]
+    r = slot_ids.numel()
+    for name, t, width in (("q", q, qk_heads * dim), ("k", k, qk_heads * dim), ("v", v, heads * vdim)):
+        _need(t.is_cuda and t.dtype == torch.float32 and t.dim() == 2 and t.shape == (n, width) and (n == 0 or t.stride(1) == 1),
+              f"{name} must be a float [n, {width}] view with unit column stride")
+    _need(heads % qk_heads == 0, "heads must be a multiple of the q/k heads")
+    _f32(decay, "decay")
+    _need(tuple(decay.shape) in ((n, heads), (heads,)), "decay must be [n, heads] or [heads]")
+    if write is not None:
+        _f32(write, "write", n * heads)
+    if skip is not None:
+        _f32(skip, "skip", heads)
+    _f32(state, "state")
+    _need(state.dim() == 4 and tuple(state.shape[1:]) == (heads, dim, vdim), "state must be [slots, heads, dim, vdim]")
+    _need(dim <= recurrence_max_dim(), f"key size {dim} above the kernel's {recurrence_max_dim()}")
+    _i32(slot_ids, "slot_ids")
+    _i32(cu_seqlens, "cu_seqlens", r + 1)
+    out = torch.empty((n, heads * vdim), dtype=torch.float32, device=v.device)
+    if n == 0:
+        return out
+    _check(library.core().jv_recurrence_steps(
+        _ptr(out), _ptr(q), c_longlong(q.stride(0)), _ptr(k), c_longlong(k.stride(0)), _ptr(v), c_longlong(v.stride(0)),
+        _ptr(decay), c_int(heads if decay.dim() == 2 else 0), _ptr(write), _ptr(skip), _ptr(state), _ptr(slot_ids),
+        _ptr(cu_seqlens), c_int(r), c_int(heads), c_int(qk_heads), c_int(dim), c_int(vdim), c_int(1 if delta else 0), _stream()),
+        "recurrence_steps")
+    return out
+
+
+NORM_GATES = {"silu": 1, "sigmoid": 2}
+
+
+def group_gated_norm(o: torch.Tensor, gate: torch.Tensor, weight, group: int, eps: float, gate_activation: str = "silu",
+                     gate_first: bool = False, out_scale: float = 1.0) -> torch.Tensor:
+    """Float rows ``o`` [n, width] normed in equal groups of ``group`` columns (each by its own root mean square), times
+    ``weight`` (float, any length that divides the width: it repeats; None: no weight), with act(gate) multiplied in
+    before the norm (``gate_first``) or behind it, times ``out_scale``; ``gate`` is a [n, width] view (unit column
+    stride) of the activation type, which is also the result's."""
+    _dev(o, weight)
+    _f32(o, "o")
+    n, width = o.shape
+    _need(group > 0 and width % group == 0, "the width must be whole groups")
+    _need(gate_activation in NORM_GATES, f"gate activation {gate_activation!r}: one of {sorted(NORM_GATES)}")
+    period = 0
+    if weight is not None:
+        _f32(weight, "weight")
+        period = weight.numel()
+        _need(period > 0 and width % period == 0, "the weight's length must divide the width")
+    _need(gate.is_cuda and gate.shape == o.shape and (n == 0 or gate.stride(1) == 1), "gate must be a [n, width] view with unit column stride")
+    out = torch.empty((n, width), dtype=gate.dtype, device=o.device)
+    fn = getattr(library.core(), f"jv_group_gated_norm_{_suffix(gate.dtype)}")
+    _check(fn(_ptr(out), _ptr(o), _ptr(gate), c_longlong(gate.stride(0) if n else 0), _ptr(weight), c_int(period), c_int(n),
+              c_int(width), c_int(group), c_float(eps), c_int(NORM_GATES[gate_activation]), c_int(1 if gate_first else 0),
+              c_float(out_scale), _stream()), "group_gated_norm")
     return out
 
 

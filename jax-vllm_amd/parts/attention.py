@@ -24,13 +24,30 @@ class GroupedQueryAttention:
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qk_norm_eps: Optional[float] = None, position: Optional[PartSpec] = None,
                  window: Optional[int] = None, scale: Optional[float] = None, qkv_bias: bool = False,
-                 o_bias: bool = False):
+                 o_bias: bool = False, v_head_dim: Optional[int] = None, qk_norm: str = "head", v_scale: float = 1.0):
+        """``v_head_dim``: a value size that differs from the key size; ``qk_norm`` "whole": the q/k norm spans all
+        of q's (and all of k's) columns at once, with weights of that size, instead of every head on its own;
+        ``v_scale``: a constant on the values (and so on the mixer's result before its output projection).  Any of
+        the three takes the ``wide`` path: heads cached under one padded size (``K.padded_head_dim``), prepared by
+        ``K.attn_prepare_wide``, read by the same paged attention kernels."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} q heads are not a multiple of {num_kv_heads} kv heads")
-        self.hidden_size, self.nq, self.nkv, self.d = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
+        if qk_norm not in ("head", "whole"):
+            raise ValueError(f"qk_norm is 'head' or 'whole', not {qk_norm!r}")
+        self.hidden_size, self.nq, self.nkv = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.dk = int(head_dim)
+        self.dv = int(v_head_dim) if v_head_dim else self.dk
+        self.qk_norm, self.v_scale = qk_norm, float(v_scale)
+        self.wide = self.dv != self.dk or (qk_norm == "whole" and qk_norm_eps is not None) or self.v_scale != 1.0
+        # what the paged attention kernels see
+        self.d = K.padded_head_dim(self.dk, self.dv) if self.wide else self.dk
+        if self.wide:
+            self.q_row_stride = self.nq * self.d
+            if qk_norm_eps is not None and qk_norm == "head":
+                raise ValueError("heads of two sizes or scaled values with a q/k norm per head: no kernel prepares that")
         self.qk_norm_eps = qk_norm_eps
         self.window = int(window) if window else None
-        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.dk)
         self.position = build_part("position", position) if position is not None else None
         # what the position part asks of this mixer's kernels: a rotation of q and k by position
         # (rotary_dim, interleaved), or nothing (a part that acts elsewhere, or no part at all)
@@ -48,18 +65,19 @@ class GroupedQueryAttention:
 
     def tensors(self) -> dict:
         t = {
-            "q_proj.weight": TensorSpec((self.nq * self.d, self.hidden_size)),
-            "k_proj.weight": TensorSpec((self.nkv * self.d, self.hidden_size)),
-            "v_proj.weight": TensorSpec((self.nkv * self.d, self.hidden_size)),
-            "o_proj.weight": TensorSpec((self.hidden_size, self.nq * self.d)),
+            "q_proj.weight": TensorSpec((self.nq * self.dk, self.hidden_size)),
+            "k_proj.weight": TensorSpec((self.nkv * self.dk, self.hidden_size)),
+            "v_proj.weight": TensorSpec((self.nkv * self.dv, self.hidden_size)),
+            "o_proj.weight": TensorSpec((self.hidden_size, self.nq * self.dv)),
         }
         if self.qk_norm_eps is not None:
-            t["q_norm.weight"] = TensorSpec((self.d,), role="vector", init="norm")
-            t["k_norm.weight"] = TensorSpec((self.d,), role="vector", init="norm")
+            whole = self.qk_norm == "whole"
+            t["q_norm.weight"] = TensorSpec((self.nq * self.dk if whole else self.dk,), role="vector", init="norm")
+            t["k_norm.weight"] = TensorSpec((self.nkv * self.dk if whole else self.dk,), role="vector", init="norm")
         if self.qkv_bias:
-            t["q_proj.bias"] = TensorSpec((self.nq * self.d,), role="vector")
-            t["k_proj.bias"] = TensorSpec((self.nkv * self.d,), role="vector")
-            t["v_proj.bias"] = TensorSpec((self.nkv * self.d,), role="vector")
+            t["q_proj.bias"] = TensorSpec((self.nq * self.dk,), role="vector")
+            t["k_proj.bias"] = TensorSpec((self.nkv * self.dk,), role="vector")
+            t["v_proj.bias"] = TensorSpec((self.nkv * self.dv,), role="vector")
         if self.o_bias:
             t["o_proj.bias"] = TensorSpec((self.hidden_size,), role="vector")
         return t
@@ -76,6 +94,11 @@ class GroupedQueryAttention:
             [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dim=0
         ).contiguous()
         self.w_o = tensors["o_proj.weight"]
+        if self.wide and self.d != self.dv:
+            # the attention's result has heads of the padded size (zeros behind the values): zero columns there
+            w = self.w_o.new_zeros((self.hidden_size, self.nq, self.d))
+            w[:, :, :self.dv] = self.w_o.view(self.hidden_size, self.nq, self.dv)
+            self.w_o = w.view(self.hidden_size, self.nq * self.d).contiguous()
         if self.qk_norm_eps is not None:
             self.q_norm, self.k_norm = tensors["q_norm.weight"], tensors["k_norm.weight"]
         if self.qkv_bias:
@@ -89,6 +112,8 @@ class GroupedQueryAttention:
         """Whether the kernel behind the qkv product (norm, rotation, page write) adds float partial
         products itself: decided by sizes and the declared rotation alone, so the same answer holds
         when the norm before asks and when the product runs."""
+        if self.wide:
+            return False
         rotary_dim, interleaved = self.rotation if self.rotation is not None else (0, False)
         return K.rope_takes_parts(self.dtype, self.d, interleaved, rotary_dim, self.rotation is not None)
 
@@ -104,6 +129,8 @@ class GroupedQueryAttention:
         # at few rows the projection may come as float partial products, which the next kernel adds
         qkv = K.linear(x, self.w_qkv, partial_max_width=None,       # the rotation kernel adds parts of any width
                        partial_ok=self._qkv_parts_ok())
+        if self.wide:
+            return self._forward_wide(qkv, ctx, mem, cos_sin, rotary_dim, interleaved)
         if self.b_qkv is not None:
             K.add_bias(qkv, self.b_qkv)
         parts = None
@@ -121,6 +148,24 @@ class GroupedQueryAttention:
 
         attention_backend.run(self, out, qkv, ctx, mem)
         y = K.linear(out, self.w_o, partial_ok=True)      # the next norm adds the partial products
+        if self.b_o is not None:
+            K.add_bias(y, self.b_o)
+        return y
+
+
+    def _forward_wide(self, qkv, ctx: StepContext, mem: LayerMemory, cos_sin, rotary_dim: int, interleaved: bool):
+        if interleaved:
+            raise ValueError("heads of two sizes and a norm over the whole projection rotate half-split pairs only")
+        writes = mem.writes
+        q = K.attn_prepare_wide(
+            qkv, self.b_qkv, self.q_norm, self.k_norm, self.qk_norm_eps or 0.0, cos_sin, rotary_dim,
+            ctx.slot_mappings[mem.group] if writes else None, mem.pages["k"] if writes else None,
+            mem.pages["v"] if writes else None, ctx.page_size, self.nq, self.nkv, self.dk, self.dv, self.d, self.v_scale)
+        out = torch.empty((qkv.shape[0], self.nq * self.d), dtype=qkv.dtype, device=qkv.device)
+        from . import attention_backend
+
+        attention_backend.run(self, out, q, ctx, mem)
+        y = K.linear(out, self.w_o, partial_ok=True)
         if self.b_o is not None:
             K.add_bias(y, self.b_o)
         return y

@@ -98,5 +98,59 @@ class SandwichBlock:
         return K.PendingNorm(*K.split_sublayer_output(f), self.norms[3].weight, self.norms[3].eps)
 
 
+class OutputNormBlock:
+    """A norm on every sublayer's OUTPUT only; the sublayers read the stream itself:
+
+        h = h + norm_1(mixer(h));   h = h + norm_2(feed_forward(h))
+
+    (the second line only for a layer that has a feed-forward; a constant factor on the sublayer's share is the
+    norm part's ``gain``).  A sublayer's output is handed on as a ``K.PendingNorm``; the kernel that norms it and adds
+    it to the float stream also hands the next reader the stream in the activation type."""
+
+    def __init__(self, norm: PartSpec, has_feed_forward: bool = True, names=("norm1", "norm2")):
+        self.has_feed_forward = bool(has_feed_forward)
+        self.names = tuple(names) if self.has_feed_forward else tuple(names[:1])
+        self.norms = [build_part("norm", norm) for _ in self.names]
+
+    @property
+    def replayable(self) -> bool:
+        return all(is_replayable(n) for n in self.norms)
+
+    def tensors(self) -> dict:
+        out = {}
+        for name, part in zip(self.names, self.norms):
+            for k, v in part.tensors().items():
+                out[f"{name}.{k}"] = v
+        return out
+
+    def bind(self, tensors: dict, dtype: torch.dtype) -> None:
+        self.dtype = dtype
+        for name, part in zip(self.names, self.norms):
+            part.bind({k[len(name) + 1:]: v for k, v in tensors.items() if k.startswith(name + ".")}, dtype)
+
+    def _stream(self, h, delta):
+        """h += (what ``delta`` still owes the stream); returns h in the activation type."""
+        from ..ops import kernels as K
+
+        if delta is None:
+            return K.cast_rows(h, self.dtype)
+        if not isinstance(delta, K.PendingNorm):
+            raise TypeError("this arrangement follows layers that hand on a sublayer's output with its norm")
+        out = torch.empty(h.shape, dtype=self.dtype, device=h.device)
+        K.postnorm_add_rmsnorm(h, delta.y, delta.parts, delta.weight, delta.eps, None, out)
+        return out
+
+    def forward(self, h, delta, mixer, feed_forward, ctx, mem):
+        from ..ops import kernels as K
+
+        a = mixer.forward(self._stream(h, delta), ctx, mem)
+        pending = K.PendingNorm(*K.split_sublayer_output(a), self.norms[0].weight, self.norms[0].eps)
+        if not self.has_feed_forward:
+            return pending
+        f = feed_forward.forward(self._stream(h, pending), ctx)
+        return K.PendingNorm(*K.split_sublayer_output(f), self.norms[1].weight, self.norms[1].eps)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "output_norm", OutputNormBlock)
 register_part("block", "sandwich", SandwichBlock)

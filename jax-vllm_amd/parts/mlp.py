@@ -45,4 +45,40 @@ class GatedMLP:
         return K.linear(z, self.w_down, partial_ok=self.partial_out)   # the next norm adds the partial products
 
 
+class DenseMLP:
+    """A feed-forward without a gate: ``down( act(up(x) + b_up) ) + b_down``; the activation is one of
+    ``ops.kernels.PLAIN_ACTIVATIONS`` ("gelu" is the erf form), computed in float; the biases are optional."""
+
+    replayable = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "gelu", bias: bool = True):
+        if activation not in K.PLAIN_ACTIVATIONS or activation is None:
+            raise ValueError(f"DenseMLP has kernels for {sorted(a for a in K.PLAIN_ACTIVATIONS if a)}, not for {activation!r}")
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.activation, self.bias = activation, bool(bias)
+        self.w_up = self.w_down = self.b_up = self.b_down = None
+
+    def tensors(self) -> dict:
+        h, i = self.hidden_size, self.intermediate_size
+        t = {"up_proj.weight": TensorSpec((i, h)), "down_proj.weight": TensorSpec((h, i))}
+        if self.bias:
+            t["up_proj.bias"] = TensorSpec((i,), role="vector")
+            t["down_proj.bias"] = TensorSpec((h,), role="vector")
+        return t
+
+    def bind(self, tensors: dict, dtype: torch.dtype) -> None:
+        self.w_up, self.w_down = tensors["up_proj.weight"], tensors["down_proj.weight"]
+        if self.bias:
+            self.b_up, self.b_down = tensors["up_proj.bias"], tensors["down_proj.bias"]
+
+    def forward(self, x, ctx=None) -> torch.Tensor:
+        z = K.linear(x, self.w_up)
+        K.bias_act(z, self.b_up, self.activation)
+        y = K.linear(z, self.w_down, partial_ok=True)       # the next norm adds the partial products
+        if self.b_down is not None:
+            K.add_bias(y, self.b_down)
+        return y
+
+
 register_part("feed_forward", "gated_mlp", GatedMLP)
+register_part("feed_forward", "dense_mlp", DenseMLP)

@@ -17,15 +17,21 @@ class RMSNorm:
     replayable = True
     may_leave_scale = True     # ``add_norm`` takes ``unscaled_ok`` (a norm part without this attribute is never asked)
 
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, one_plus: bool = False, gain: float = 1.0):
+        """``one_plus``: the stored weight lies around zero and the norm multiplies by 1 + weight.  ``gain``: a
+        constant factor on the result (a residual multiplier folded into the norm of a sublayer's output)."""
         self.size, self.eps = int(size), float(eps)
+        self.one_plus, self.gain = bool(one_plus), float(gain)
         self.weight = None
 
     def tensors(self) -> dict:
-        return {"weight": TensorSpec((self.size,), role="vector", init="norm")}
+        return {"weight": TensorSpec((self.size,), role="vector", init="small" if self.one_plus else "norm")}
 
     def bind(self, tensors: dict, dtype: torch.dtype) -> None:
-        self.weight = tensors["weight"]
+        w = tensors["weight"]
+        if self.one_plus or self.gain != 1.0:
+            w = ((w + 1.0 if self.one_plus else w) * self.gain).contiguous()     # float: the kernels see one weight
+        self.weight = w
         self.dtype = dtype
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:

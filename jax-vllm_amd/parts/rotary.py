@@ -22,7 +22,7 @@ class RotaryEncoding:
     replayable = True      # the table is computed on the device from the step's positions
 
     def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None, interleaved: bool = False,
-                 rescale: dict | None = None):
+                 rescale: dict | None = None, by_wavelength: dict | None = None):
         self.head_dim = int(head_dim)
         self.theta = float(theta)
         self.rotary_dim = int(rotary_dim) if rotary_dim is not None else self.head_dim
@@ -32,6 +32,10 @@ class RotaryEncoding:
         # frequencies rescaled for contexts longer than the ``original`` one (YaRN): see ``inverse_frequencies``
         self.rescale = dict(rescale) if rescale else None
         self.amplitude = 0.1 * math.log(float(self.rescale["factor"])) + 1.0 if self.rescale else 1.0
+        # frequencies slowed down by wavelength (the Llama 3.1 rule): see ``inverse_frequencies``
+        self.by_wavelength = dict(by_wavelength) if by_wavelength else None
+        if self.rescale and self.by_wavelength:
+            raise ValueError("one rule for the frequencies, not two")
         self.inv_freq = None
 
     def tensors(self) -> dict:
@@ -40,6 +44,17 @@ class RotaryEncoding:
     def inverse_frequencies(self) -> torch.Tensor:
         """float32 table of rotary_dim/2 entries, computed as the reference does."""
         d = self.rotary_dim
+        if self.by_wavelength is not None:
+            # ``by_wavelength`` = {factor, low, high, original}: a pair whose wavelength 2 pi / f is below original / high
+            # keeps f, one above original / low turns ``factor`` times slower, and between the two f is blended with
+            # f / factor by s = (original / wavelength - low) / (high - low).  Computed in double, rounded once.
+            r = {k: float(v) for k, v in self.by_wavelength.items()}
+            f = self.theta ** (-2.0 * torch.arange(d // 2, dtype=torch.float64) / d)
+            wave = 2 * math.pi / f
+            s = (r["original"] / wave - r["low"]) / (r["high"] - r["low"])
+            out = torch.where(wave < r["original"] / r["high"], f,
+                              torch.where(wave > r["original"] / r["low"], f / r["factor"], (1 - s) * f / r["factor"] + s * f))
+            return out.to(torch.float32)
         if self.rescale is None:
             return 1.0 / (self.theta ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
         # With ``rescale`` = {factor, original, fast, slow}: a pair that makes more than ``fast`` turns over
@@ -69,7 +84,8 @@ class RotaryEncoding:
 
     def rotation_table(self, ctx):
         """Float cos/sin table of the step's positions for the attention-input kernel."""
-        key = ("rope_table", self.theta, self.rotary_dim, tuple(sorted(self.rescale.items())) if self.rescale else None)
+        key = ("rope_table", self.theta, self.rotary_dim, tuple(sorted(self.rescale.items())) if self.rescale else None,
+               tuple(sorted(self.by_wavelength.items())) if self.by_wavelength else None)
         table = ctx.extras.get(key)
         if table is None:
             if self.rescale is None:

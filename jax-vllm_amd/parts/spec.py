@@ -24,8 +24,8 @@ class TensorSpec:
            "vector"  – a small floating tensor always held in float32 (norm weights and the like:
                         a checkpoint's 32-bit values stay 32-bit, 16-bit values widen exactly);
            "table"   – an integer table, held as int32.
-    init:  how the random-weights mode fills it: "normal" N(0, std), "norm" 1 + N(0, norm_std),
-           "zeros", or "index" (0, 1, 2, ... for integer tables).
+    init:  how the random-weights mode fills it: "normal" N(0, std), "norm" 1 + N(0, norm_std), "small"
+           N(0, norm_std), "log_rate" -3 + N(0, 1), "zeros", or "index" (0, 1, 2, ... for integer tables).
     """
 
     shape: tuple
@@ -101,10 +101,24 @@ def kv_cache_spec(num_kv_heads: int, head_dim: int, window: Optional[int] = None
 
 @dataclass(frozen=True)
 class StateSpec:
-    """State of fixed size per request (one row per slot), zeroed when a request starts."""
+    """State of fixed size per request (one row per slot), zeroed when a request starts.  A mixer that
+    keeps several such tensors (a recurrence's matrix and the last inputs of a short convolution, say)
+    returns a tuple of them from ``state_spec()``, each with a ``name`` of its own."""
 
     shape: tuple
     dtype: str = "float32"
+    name: str = "state"
+
+
+def state_specs_of(spec) -> tuple:
+    """What ``state_spec()`` returned as a tuple of ``StateSpec`` with distinct names (empty for None)."""
+    if spec is None:
+        return ()
+    specs = (spec,) if isinstance(spec, StateSpec) else tuple(spec)
+    names = [s.name for s in specs]
+    if len(set(names)) != len(names):
+        raise ValueError(f"a mixer's state tensors need distinct names, got {names}")
+    return specs
 
 
 @dataclass
@@ -114,14 +128,22 @@ class LayerMemory:
     ``pages``: the storage of every tensor the run's mixer declared in its ``PagedCacheSpec``, by
     name, each ``[pages + 1, *page_shape]`` (empty for a mixer without a paged cache);
     ``group`` says which block table / slot mapping of the step applies; ``writes`` is False for
-    a run that reads another run's cache.  ``state`` is [slots + 1, *shape] or None; its last row
-    belongs to no request (rows that pad a captured step point there).
+    a run that reads another run's cache.  ``states``: every state tensor the mixer declared, by
+    name, each [slots + 1, *shape]; the last row belongs to no request (rows that pad a captured step
+    point there).  ``state`` is the first of them (the only one of most mixers) or None.
     """
 
     pages: dict = field(default_factory=dict)
     group: int = 0
     writes: bool = True
     state: Optional[torch.Tensor] = None
+    states: dict = field(default_factory=dict)
+
+    def below(self, prefix: str) -> "LayerMemory":
+        """The memory of a mixer inside this one whose state names were declared with ``prefix`` in front:
+        the same pages and group, the states of that prefix under their own names."""
+        own = {k[len(prefix):]: v for k, v in self.states.items() if k.startswith(prefix)}
+        return LayerMemory(self.pages, self.group, self.writes, next(iter(own.values()), None), own)
 
 
 @dataclass

@@ -31,6 +31,10 @@ def _draw(ts, seed: int, name: str, std: float, norm_std: float, device="cpu") -
         return torch.randn(ts.shape, generator=g, dtype=torch.float32, device=device) * std
     if ts.init == "norm":
         return 1.0 + torch.randn(ts.shape, generator=g, dtype=torch.float32, device=device) * norm_std
+    if ts.init == "small":        # a weight stored around zero (a norm that multiplies by 1 + weight)
+        return torch.randn(ts.shape, generator=g, dtype=torch.float32, device=device) * norm_std
+    if ts.init == "log_rate":     # the logarithm of a decay rate: rates around e^-3, a factor e either way
+        return torch.randn(ts.shape, generator=g, dtype=torch.float32, device=device) - 3.0
     if ts.init == "zeros":
         return torch.zeros(ts.shape, dtype=torch.float32, device=device)
     if ts.init == "index":
