@@ -3,6 +3,7 @@ prefill tokens/s at 2,048 tokens and decode at batch 1 and 64 beside it.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--shape 8b|14b|32b]
     python bench.py --only design [--design-shape 2k|4k]     # the Lomozen architecture beside the dense model of equal size
+    python bench.py --only design --design dumazen           # the Dumazen architecture beside Lomozen and the dense model
 
 The model has the layer sizes of Qwen3-8B (the headline configuration) with random
 weights drawn on the device; prompts are seeded uniform-random token ids of 1,024 tokens;
@@ -54,6 +55,22 @@ def lomozen_shape(width, layers, heads, experts, top, expert_ff, shared_ff, voca
             "layers": [dict(lightning if i % 4 == 0 else latent, mlp=mlp) for i in range(layers)]}
 
 
+def dumazen_shape(width, layers, heads, ff, vocab=32000, window=1024):
+    """Layers in the order retention, state-space, (window attention beside the gated delta rule), state-space, with
+    heads of 128 (state-space: heads of 64 over twice the width, a state of 128, as published models of that kind
+    have), a dense feed-forward in every layer."""
+    retention = {"type": "retention", "mixer": {"heads": heads, "dim": 128, "vdim": 128, "rot": {"base": 1e6, "dims": 128},
+                                                "decay": [1.0 - 2.0 ** (-5 - 3 * h / heads) for h in range(heads)]}}
+    mamba2 = {"type": "mamba2", "mixer": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 1, "norm_groups": 1, "conv": 4}}
+    left = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": window},
+            "rot": {"base": 1e6, "dims": 128, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    right = {"heads": heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4}
+    par = {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 0.6, "right_scale": 0.9}}
+    order = (retention, mamba2, par, mamba2)
+    return {"architecture": "Dumazen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.7,
+            "layers": [dict(order[i % 4], mlp={"kind": "dense", "ff": ff}) for i in range(layers)]}
+
+
 # --only design: Lomozen beside the dense model of the same width, depth, vocabulary and feed-forward
 # parameters per token (top * expert + shared = intermediate)
 DESIGN_SHAPES = {
@@ -63,6 +80,12 @@ DESIGN_SHAPES = {
     "4k": (lomozen_shape(4096, 8, 32, 64, 6, 1024, 2048),
            dict(QWEN3_8B, num_hidden_layers=8, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
                 head_dim=128, intermediate_size=8192, vocab_size=32000)),
+}
+# --only design --design dumazen: Dumazen beside Lomozen (the closest kin: linear attention with a state, attention inside
+# a window) and the dense model, all of one width, depth and vocabulary (feed-forward parameters per token: 2 * ff = 3 * intermediate)
+DUMAZEN_SHAPES = {
+    "2k": (dumazen_shape(2048, 8, 16, 4608),) + DESIGN_SHAPES["2k"],
+    "4k": (dumazen_shape(4096, 8, 32, 12288),) + DESIGN_SHAPES["4k"],
 }
 PROMPT_LEN = 1024
 MAX_CONTEXT = 8192
@@ -188,7 +211,12 @@ def measure_design(args, rng):
     from jax_vllm_amd.engine.entries import StepEntry
 
     out = {"shape": args.design_shape, "dtype": args.dtype, "prefill_tokens": PREFILL_TOKENS, "decode_prompt_len": PROMPT_LEN}
-    for name, cfg in zip(("lomozen", "dense"), DESIGN_SHAPES[args.design_shape]):
+    models = (zip(("dumazen", "lomozen", "dense"), DUMAZEN_SHAPES[args.design_shape]) if args.design == "dumazen"
+              else zip(("lomozen", "dense"), DESIGN_SHAPES[args.design_shape]))
+    out["design"] = args.design
+    for name, cfg in models:
+        if args.design_models and name not in args.design_models.split(","):
+            continue
         vocab = cfg.get("vocab") or cfg["vocab_size"]
         llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=16, max_num_seqs=32, max_model_len=4096,
                   num_blocks=1 + 32 * (2048 // 16) + 256, max_num_batched_tokens=PREFILL_TOKENS, enable_prefix_cache=False)
@@ -353,6 +381,9 @@ def main():
     ap.add_argument("--no-kernel-share", action="store_true", help="leave out the per-kernel time shares")
     ap.add_argument("--design-shape", choices=sorted(DESIGN_SHAPES), default="2k",
                     help="with --only design: the width of both models (2,048 or 4,096), 8 layers each")
+    ap.add_argument("--design", choices=["lomozen", "dumazen"], default="lomozen",
+                    help="with --only design: the architecture that is measured beside its kin of equal size")
+    ap.add_argument("--design-models", default="", help="with --only design: only these of the models, with commas between them")
     ap.add_argument("--only", choices=["prefill", "decode", "mixed", "long-prompt", "ttft", "calibrate", "design"], default=None,
                     help="run one phase alone and print its result (for profiling); mixed: 32 running decodes "
                          "joined by 4 prompts of 3,000 tokens in portions of 512 under a budget of 2,048; "

@@ -217,6 +217,246 @@ recurrence_steps_kernel(float* __restrict__ out, const float* __restrict__ q, lo
   }
 }
 
+// ---------------------------------------------------------------- the recurrence by chunks (delta = 0)
+// With c_i = sum_{m <= i} log g_m inside a chunk of n <= RC_LC tokens and S0 the state before it:
+//     o_i   = exp(c_i) S0^T q_i + sum_{j <= i} exp(c_i - c_j) (q_i . k_j) w_j v_j  (+ skip v_i)
+//     S_end = exp(c_(n-1)) S0 + sum_j exp(c_(n-1) - c_j) w_j k_j v_j^T
+// Only differences c_i - c_j <= 0 are exponentiated (a decay of 0 counts as 1e-38).  Three launches, so that the
+// chunks of a long prompt run side by side and only the cheap part is serial:
+//   local:  per (chunk, head, slice)  out_i = sum_j a[i][j] v_j;  U = sum_j k'_j v_j^T -> scratch[chunk];  exp(c_i) -> cum
+//   scan:   per (request, head)       for its chunks in order: scratch[chunk] <- S (the state BEFORE the chunk),
+//                                     S <- exp(c_(n-1)) S + U;  at the end state <- S
+//   apply:  per (chunk, head, slice)  out_i += exp(c_i) S_before^T q_i
+#define RC_LC 32        // tokens of a chunk
+#define RC_LV 128       // columns (elements of v) a block takes
+#define RC_PAD 4        // row padding of q and k in LDS: rows stay 16-byte aligned
+
+// grid (chunks, heads, column slices of RC_LV); work: chunk -> (request, first token)
+__global__ void __launch_bounds__(256)
+recurrence_local_kernel(float* __restrict__ out, float* __restrict__ scratch, float* __restrict__ cum,
+                        const float* __restrict__ q, long long ldq, const float* __restrict__ k, long long ldk,
+                        const float* __restrict__ v, long long ldv, const float* __restrict__ g, int g_stride,
+                        const float* __restrict__ wgt, const float* __restrict__ skip, const int* __restrict__ work,
+                        const int* __restrict__ cu_seqlens, int heads, int qk_heads, int dim, int vdim) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int ch = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * RC_LV;
+  const int r = work[2 * ch], b0 = work[2 * ch + 1];
+  const int n = min(RC_LC, cu_seqlens[r + 1] - b0);
+  const int hk = h / (heads / qk_heads);
+  const int dq = dim + RC_PAD;
+  float* qs = lds;                       // [LC][dq]
+  float* ks = qs + RC_LC * dq;           // [LC][dq]
+  float* vs = ks + RC_LC * dq;           // [LC][LV]
+  float* as = vs + RC_LC * RC_LV;        // [LC][LC + 1]
+  float* cl = as + RC_LC * (RC_LC + 1);  // [LC] cumulative log decay
+  float* ws = cl + RC_LC;                // [LC] write strengths
+  const int tid = threadIdx.x;
+  const int ncols = min(RC_LV, vdim - c0);
+  if (tid < RC_LC) {
+    float lg = 0.f, w = 0.f;
+    if (tid < n) {
+      lg = logf(fmaxf(g[(long long)(b0 + tid) * g_stride + h], 1e-38f));
+      w = wgt ? wgt[(long long)(b0 + tid) * heads + h] : 1.f;
+    }
+    // inclusive prefix sum over the first 32 lanes of wave 0
+#pragma unroll
+    for (int o = 1; o < RC_LC; o <<= 1) {
+      const float up = __shfl_up(lg, o, JV_WAVE);
+      if (tid >= o) lg += up;
+    }
+    cl[tid] = lg;
+    ws[tid] = w;
+    if (blockIdx.z == 0 && tid < n) cum[(long long)(b0 + tid) * heads + h] = expf(lg);
+  }
+  for (int i = tid; i < RC_LC * dq; i += 256) {
+    const int j = i / dq, d = i - j * dq;
+    float qv = 0.f, kv = 0.f;
+    if (j < n && d < dim) {
+      qv = q[(long long)(b0 + j) * ldq + hk * dim + d];
+      kv = k[(long long)(b0 + j) * ldk + hk * dim + d];
+    }
+    qs[i] = qv;
+    ks[i] = kv;
+  }
+  for (int i = tid; i < RC_LC * RC_LV; i += 256) {
+    const int j = i / RC_LV, c = i % RC_LV;
+    vs[i] = (j < n && c < ncols) ? v[(long long)(b0 + j) * ldv + h * vdim + c0 + c] : 0.f;
+  }
+  __syncthreads();
+  // a: thread (i, 4 consecutive j)
+  {
+    const int i = tid >> 3, j0 = (tid & 7) * 4;
+    float dot[4] = {0.f, 0.f, 0.f, 0.f};
+    if (j0 <= i) {
+      for (int d = 0; d < dim; ++d) {
+        const float qv = qs[i * dq + d];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) dot[u] = fmaf(qv, ks[(j0 + u) * dq + d], dot[u]);
+      }
+    }
+    const float sk = skip ? skip[h] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u;
+      float a = 0.f;
+      if (j <= i && i < n) a = dot[u] * expf(cl[i] - cl[j]) * ws[j] + (j == i ? sk : 0.f);
+      as[i * (RC_LC + 1) + j] = a;
+    }
+  }
+  __syncthreads();
+  // k_j <- exp(c_(n-1) - c_j) w_j k_j (rows beyond the chunk are zero already); out = a v
+  for (int i = tid; i < RC_LC * dq; i += 256) {
+    const int j = i / dq;
+    if (j < n) ks[i] *= expf(cl[n - 1] - cl[j]) * ws[j];
+  }
+  for (int e = tid; e < RC_LC * (RC_LV / 4); e += 256) {
+    const int i = e / (RC_LV / 4), c = (e % (RC_LV / 4)) * 4;
+    if (i < n && c < ncols) {
+      float4 o = {0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j <= i; ++j) {
+        const float a = as[i * (RC_LC + 1) + j];
+        const float4 x = *(const float4*)(vs + j * RC_LV + c);
+        o.x = fmaf(a, x.x, o.x); o.y = fmaf(a, x.y, o.y); o.z = fmaf(a, x.z, o.z); o.w = fmaf(a, x.w, o.w);
+      }
+      float* dst = out + (long long)(b0 + i) * heads * vdim + h * vdim + c0 + c;
+      dst[0] = o.x;
+      if (c + 1 < ncols) dst[1] = o.y;
+      if (c + 2 < ncols) dst[2] = o.z;
+      if (c + 3 < ncols) dst[3] = o.w;
+    }
+  }
+  __syncthreads();
+  // U[d][c]: tiles of 4 x 4 per thread
+  float* U = scratch + (((long long)ch * heads + h) * dim) * vdim + c0;
+  const int dt = (dim + 3) / 4;
+  for (int e = tid; e < dt * (RC_LV / 4); e += 256) {
+    const int d0 = (e / (RC_LV / 4)) * 4, c = (e % (RC_LV / 4)) * 4;
+    if (c >= ncols) continue;
+    float u[4][4] = {};
+    for (int j = 0; j < n; ++j) {
+      const float4 kv = *(const float4*)(ks + j * dq + d0);
+      const float4 x = *(const float4*)(vs + j * RC_LV + c);
+      const float kk[4] = {kv.x, kv.y, kv.z, kv.w}, vv[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) u[a][b] = fmaf(kk[a], vv[b], u[a][b]);
+    }
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+      if (d0 + a < dim)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          if (c + b < ncols) U[(long long)(d0 + a) * vdim + c + b] = u[a][b];
+  }
+}
+
+// grid (requests, heads, slices of the dim x vdim elements); req_chunks [requests + 1]: first chunk of each request
+__global__ void __launch_bounds__(256)
+recurrence_scan_kernel(float* __restrict__ scratch, float* __restrict__ state, const float* __restrict__ cum,
+                       const int* __restrict__ slot_ids, const int* __restrict__ req_chunks,
+                       const int* __restrict__ work, const int* __restrict__ cu_seqlens, int heads, int dim, int vdim) {
+  const int r = blockIdx.x, h = blockIdx.y;
+  const int first = req_chunks[r], last = req_chunks[r + 1];
+  if (last <= first) return;
+  const int e = blockIdx.z * 256 + threadIdx.x;
+  if (e >= dim * vdim) return;
+  float* S = state + ((long long)slot_ids[r] * heads + h) * dim * vdim + e;
+  float s = *S;
+  const int end = cu_seqlens[r + 1];
+  float next = scratch[((long long)first * heads + h) * dim * vdim + e];
+  for (int ch = first; ch < last; ++ch) {
+    float* U = scratch + ((long long)ch * heads + h) * dim * vdim + e;
+    const float u = next;
+    if (ch + 1 < last) next = U[(long long)heads * dim * vdim];     // asked for before this chunk's store
+    *U = s;
+    const int b0 = work[2 * ch + 1];
+    const int n = min(RC_LC, end - b0);
+    s = fmaf(cum[(long long)(b0 + n - 1) * heads + h], s, u);
+  }
+  *S = s;
+}
+
+// grid as the local kernel
+__global__ void __launch_bounds__(256)
+recurrence_apply_kernel(float* __restrict__ out, const float* __restrict__ scratch, const float* __restrict__ cum,
+                        const float* __restrict__ q, long long ldq, const int* __restrict__ work,
+                        const int* __restrict__ cu_seqlens, int heads, int qk_heads, int dim, int vdim) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int ch = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * RC_LV;
+  const int r = work[2 * ch], b0 = work[2 * ch + 1];
+  const int n = min(RC_LC, cu_seqlens[r + 1] - b0);
+  const int hk = h / (heads / qk_heads);
+  const int dq = dim + 1;
+  float* qs = lds;                       // [LC][dq]
+  float* ps = qs + RC_LC * dq;           // [32][LV]: a slab of 32 rows of the state
+  const int tid = threadIdx.x;
+  const int ncols = min(RC_LV, vdim - c0);
+  for (int i = tid; i < RC_LC * dim; i += 256) {
+    const int j = i / dim, d = i - j * dim;
+    qs[j * dq + d] = j < n ? q[(long long)(b0 + j) * ldq + hk * dim + d] : 0.f;
+  }
+  const float* P = scratch + (((long long)ch * heads + h) * dim) * vdim + c0;
+  const int i0 = (tid >> 5) * 4, c = (tid & 31) * 4;       // thread: rows i0..i0+3, columns c..c+3
+  float o[4][4] = {};
+  for (int d0 = 0; d0 < dim; d0 += 32) {
+    __syncthreads();
+    for (int e = tid; e < 32 * RC_LV; e += 256) {
+      const int d = d0 + e / RC_LV, cc = e % RC_LV;
+      ps[e] = (d < dim && cc < ncols) ? P[(long long)d * vdim + cc] : 0.f;
+    }
+    __syncthreads();
+    const int dn = min(32, dim - d0);
+    for (int d = 0; d < dn; ++d) {
+      const float4 p = *(const float4*)(ps + d * RC_LV + c);
+      const float pp[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const float qv = qs[(i0 + a) * dq + d0 + d];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) o[a][b] = fmaf(qv, pp[b], o[a][b]);
+      }
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int i = i0 + a;
+    if (i >= n) continue;
+    const float w = cum[(long long)(b0 + i) * heads + h];
+    float* dst = out + (long long)(b0 + i) * heads * vdim + h * vdim + c0 + c;
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+      if (c + b < ncols) dst[b] += w * o[a][b];
+  }
+}
+
+extern "C" int jv_recurrence_chunk_tokens() { return RC_LC; }
+extern "C" int jv_recurrence_chunk_max_dim() { return 128; }
+
+// work [chunks][2] = (request, first token) in the order of requests and tokens, req_chunks [requests + 1], scratch of
+// chunks * heads * dim * vdim floats, cum of tokens * heads floats.
+extern "C" int jv_recurrence_chunks(float* out, const float* q, long long ldq, const float* k, long long ldk,
+                                    const float* v, long long ldv, const float* g, int g_stride, const float* wgt,
+                                    const float* skip, float* state, const int* slot_ids, const int* cu_seqlens,
+                                    int n_requests, int heads, int qk_heads, int dim, int vdim, int chunks,
+                                    const int* work, const int* req_chunks, float* scratch, float* cum, void* stream) {
+  if (n_requests <= 0 || heads <= 0 || chunks <= 0) return 0;
+  if (dim <= 0 || dim > 128 || dim % 4 || vdim <= 0 || heads > 65535 || qk_heads <= 0 || heads % qk_heads || !work ||
+      !req_chunks || !scratch || !cum)
+    return (int)hipErrorInvalidValue;
+  hipStream_t s = (hipStream_t)stream;
+  const int slices = (vdim + RC_LV - 1) / RC_LV;
+  const size_t lds_local = (2 * RC_LC * (dim + RC_PAD) + RC_LC * RC_LV + RC_LC * (RC_LC + 1) + 2 * RC_LC) * sizeof(float);
+  const size_t lds_apply = (RC_LC * (dim + 1) + 32 * RC_LV) * sizeof(float);
+  hipLaunchKernelGGL(recurrence_local_kernel, dim3(chunks, heads, slices), dim3(256), lds_local, s, out, scratch, cum, q,
+                     ldq, k, ldk, v, ldv, g, g_stride, wgt, skip, work, cu_seqlens, heads, qk_heads, dim, vdim);
+  hipLaunchKernelGGL(recurrence_scan_kernel, dim3(n_requests, heads, (dim * vdim + 255) / 256), dim3(256), 0, s, scratch,
+                     state, cum, slot_ids, req_chunks, work, cu_seqlens, heads, dim, vdim);
+  hipLaunchKernelGGL(recurrence_apply_kernel, dim3(chunks, heads, slices), dim3(256), lds_apply, s, out, scratch, cum, q,
+                     ldq, work, cu_seqlens, heads, qk_heads, dim, vdim);
+  return JV_LAUNCH_CHECK();
+}
+
 // ---------------------------------------------------------------- norm in groups with a gate
 //   a = gate_first ? o * act(gate) : o;   y = a * rsqrt(mean_group(a^2) + eps) * w[c % w_period];
 //   out = T( (gate_first ? y : y * act(gate)) * out_scale );   act: 1 silu, 2 sigmoid;  w null: no weight
@@ -243,6 +483,36 @@ group_gated_norm_kernel(T* __restrict__ out, const float* __restrict__ o, const 
   ss = wave_sum(ss);
   const float inv = rsqrtf(ss / (float)group + eps) * out_scale;
   for (int i = lane; i < group; i += JV_WAVE) {
+    const float z = to_f32(gp[i]);
+    const float ga = gate_act == 1 ? rc_silu(z) : 1.f / (1.f + expf(-z));
+    const float wv = w ? w[(grp * group + i) % w_period] : 1.f;
+    out[t * width + grp * group + i] = from_f32<T>(x[i] * ga * inv * wv);
+  }
+}
+
+// The same for wide groups: one block a (row, group).
+template <typename T>
+__global__ void __launch_bounds__(256)
+group_gated_norm_block_kernel(T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ gate,
+                              long long g_stride, const float* __restrict__ w, int w_period, int width, int group,
+                              float eps, int gate_act, int gate_first, float out_scale) {
+  __shared__ float red[32];
+  const long long t = blockIdx.x;
+  const int grp = blockIdx.y;
+  const float* x = o + t * width + grp * group;
+  const T* gp = gate + t * g_stride + grp * group;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < group; i += blockDim.x) {
+    float a = x[i];
+    if (gate_first) {
+      const float z = to_f32(gp[i]);
+      a *= gate_act == 1 ? rc_silu(z) : 1.f / (1.f + expf(-z));
+    }
+    ss = fmaf(a, a, ss);
+  }
+  ss = block_sum(ss, red);
+  const float inv = rsqrtf(ss / (float)group + eps) * out_scale;
+  for (int i = threadIdx.x; i < group; i += blockDim.x) {
     const float z = to_f32(gp[i]);
     const float ga = gate_act == 1 ? rc_silu(z) : 1.f / (1.f + expf(-z));
     const float wv = w ? w[(grp * group + i) % w_period] : 1.f;
@@ -320,7 +590,13 @@ extern "C" int jv_recurrence_steps(float* out, const float* q, long long ldq, co
     if (group <= 0 || width % group || (w && w_period <= 0) || (gate_act != 1 && gate_act != 2))               \
       return (int)hipErrorInvalidValue;                                                                        \
     const int groups = width / group;                                                                          \
-    if (groups > 4 * 65535) return (int)hipErrorInvalidValue;                                                  \
+    if (groups > 65535) return (int)hipErrorInvalidValue;                                                      \
+    if (group >= 256) {                                                                                        \
+      hipLaunchKernelGGL(group_gated_norm_block_kernel<T>, dim3(n, groups), dim3(256), 0, (hipStream_t)stream, \
+                         (T*)out, o, (const T*)gate, g_stride, w, w_period, width, group, eps, gate_act,       \
+                         gate_first, out_scale);                                                               \
+      return JV_LAUNCH_CHECK();                                                                                \
+    }                                                                                                          \
     hipLaunchKernelGGL(group_gated_norm_kernel<T>, dim3(n, (groups + 3) / 4), dim3(256), 0,                    \
                        (hipStream_t)stream, (T*)out, o, (const T*)gate, g_stride, w, w_period, width, group,   \
                        eps, gate_act, gate_first, out_scale);                                                  \

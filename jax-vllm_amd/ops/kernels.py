@@ -1159,14 +1159,16 @@ def head_unit_norm(x: torch.Tensor, heads: int, d: int, eps: float, scale: float
 
 
 def recurrence_steps(q, k, v, decay, state, slot_ids, cu_seqlens, heads: int, qk_heads: int, dim: int, vdim: int,
-                     write=None, skip=None, delta: bool = False) -> torch.Tensor:
+                     write=None, skip=None, delta: bool = False, chunk_plan=None) -> torch.Tensor:
     """Float [n, heads * vdim], token by token per request and head, S [dim, vdim] float in the request's state row:
 
         S <- g S;   u = w (v - S^T k) if ``delta`` else w v;   S <- S + k u^T;   o = S^T q + skip[h] v
 
     ``q``, ``k``: float views [n, qk_heads * dim] (unit column stride; head h reads q/k head h // (heads // qk_heads)),
     ``v`` a float view [n, heads * vdim]; ``decay`` g: float [n, heads] or [heads] (constant per head); ``write`` w:
-    float [n, heads] or None (1); ``skip``: float [heads] or None."""
+    float [n, heads] or None (1); ``skip``: float [heads] or None.  ``chunk_plan`` (``recurrence_chunk_plan`` of the
+    step's token counts; not for ``delta``): the kernels that take a request's tokens a chunk at a time, chunks side
+    by side, instead of one by one (the same numbers in another order of operations)."""
     _dev(decay, write, skip, state, slot_ids, cu_seqlens)
     n = v.shape[0]
     r = slot_ids.numel()
@@ -1188,12 +1190,63 @@ def recurrence_steps(q, k, v, decay, state, slot_ids, cu_seqlens, heads: int, qk
     out = torch.empty((n, heads * vdim), dtype=torch.float32, device=v.device)
     if n == 0:
         return out
+    if chunk_plan is not None:
+        work, first, chunks = chunk_plan
+        _need(recurrence_chunks_possible(dim, delta), "the kernels by chunks take key sizes that are multiples of 4, at most 128, and no delta rule")
+        _dev(work, first)
+        _i32(work, "work", 2 * chunks)
+        _i32(first, "first chunks", r + 1)
+        scratch = torch.empty(chunks * heads * dim * vdim, dtype=torch.float32, device=v.device)
+        cum = torch.empty(n * heads, dtype=torch.float32, device=v.device)
+        _check(library.core().jv_recurrence_chunks(
+            _ptr(out), _ptr(q), c_longlong(q.stride(0)), _ptr(k), c_longlong(k.stride(0)), _ptr(v), c_longlong(v.stride(0)),
+            _ptr(decay), c_int(heads if decay.dim() == 2 else 0), _ptr(write), _ptr(skip), _ptr(state), _ptr(slot_ids),
+            _ptr(cu_seqlens), c_int(r), c_int(heads), c_int(qk_heads), c_int(dim), c_int(vdim), c_int(chunks), _ptr(work),
+            _ptr(first), _ptr(scratch), _ptr(cum), _stream()), "recurrence_chunks")
+        return out
     _check(library.core().jv_recurrence_steps(
         _ptr(out), _ptr(q), c_longlong(q.stride(0)), _ptr(k), c_longlong(k.stride(0)), _ptr(v), c_longlong(v.stride(0)),
         _ptr(decay), c_int(heads if decay.dim() == 2 else 0), _ptr(write), _ptr(skip), _ptr(state), _ptr(slot_ids),
         _ptr(cu_seqlens), c_int(r), c_int(heads), c_int(qk_heads), c_int(dim), c_int(vdim), c_int(1 if delta else 0), _stream()),
         "recurrence_steps")
     return out
+
+
+RECURRENCE_CHUNK_MIN_TOKENS = 8     # from this many tokens of a request on, the kernels by chunks
+
+
+def recurrence_chunk_tokens() -> int:
+    return library.core().jv_recurrence_chunk_tokens()
+
+
+def recurrence_chunks_possible(dim: int, delta: bool = False) -> bool:
+    """The kernels by chunks keep a chunk's keys in LDS in 16-byte pieces; the delta rule runs token by token."""
+    return not delta and dim % 4 == 0 and dim <= library.core().jv_recurrence_chunk_max_dim()
+
+
+def recurrence_chunk_plan(q_lens, device):
+    """(work int32 [chunks, 2] = (request, first token row), first chunk of every request int32 [requests + 1],
+    chunks) for the recurrence by chunks: every request's tokens of this step cut into chunks, in order."""
+    size = recurrence_chunk_tokens()
+    work, first, at = [], [0], 0
+    for r, n in enumerate(q_lens):
+        work += [(r, at + b) for b in range(0, n, size)]
+        first.append(len(work))
+        at += n
+    flat = torch.tensor([x for w in work for x in w] + first, dtype=torch.int32).pin_memory().to(device, non_blocking=True)
+    return flat[:2 * len(work)], flat[2 * len(work):], len(work)
+
+
+def step_chunk_plan(ctx, dim: int, delta: bool = False):
+    """The chunk plan of a step for a recurrence with keys of ``dim`` elements, or None where the step runs token by
+    token: a recorded step, a step of short portions only, sizes the kernels by chunks are not built for.  One plan
+    serves every such layer of the step (``ctx.plans``)."""
+    if ctx.captured or ctx.max_q_len < RECURRENCE_CHUNK_MIN_TOKENS or not recurrence_chunks_possible(dim, delta):
+        return None
+    plan = ctx.plans.get("recurrence_chunks")
+    if plan is None:
+        plan = ctx.plans["recurrence_chunks"] = recurrence_chunk_plan(ctx.q_lens_host, ctx.positions.device)
+    return plan
 
 
 NORM_GATES = {"silu": 1, "sigmoid": 2}

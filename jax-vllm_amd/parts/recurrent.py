@@ -76,13 +76,14 @@ class Retention:
         q = K.heads_to_f32(proj, 0, H, d, self.rot_dims, cos_sin)
         k = K.heads_to_f32(proj, H * d, H, d, self.rot_dims, cos_sin, scale=d ** -0.5)
         v = K.heads_to_f32(proj, 2 * H * d, H, dv)
-        o = K.recurrence_steps(q, k, v, self.decay, mem.states["S"], ctx.slot_ids, ctx.cu_seqlens, H, H, d, dv)
+        o = K.recurrence_steps(q, k, v, self.decay, mem.states["S"], ctx.slot_ids, ctx.cu_seqlens, H, H, d, dv,
+                               chunk_plan=K.step_chunk_plan(ctx, d))
         y = K.group_gated_norm(o, proj[:, 2 * H * d + H * dv:], None, dv, self.eps, "silu", out_scale=self.out_scale)
         return K.linear(y, self.w_o, partial_ok=True)
 
 
 class StateSpaceMixer:
-    replayable = True
+    replayable = True     # slots, request borders and tokens come from the device; the kernel choice does not depend on values
 
     def __init__(self, hidden_size: int, num_heads: int, v_dim: int, state_size: int, groups: int, conv_taps: int,
                  norm_groups: int, norm_eps: float, out_scale: float = 1.0):
@@ -129,7 +130,8 @@ class StateSpaceMixer:
                            ctx.cu_seqlens, ctx.max_q_len)
         g, dt = K.recurrence_gates(proj, inner + self.channels, self.dt_bias, self.a_log, H)
         v, b, c = xbc[:, :inner], xbc[:, inner:inner + G * N], xbc[:, inner + G * N:]
-        o = K.recurrence_steps(c, b, v, g, mem.states["S"], ctx.slot_ids, ctx.cu_seqlens, H, G, N, dv, write=dt, skip=self.skip)
+        o = K.recurrence_steps(c, b, v, g, mem.states["S"], ctx.slot_ids, ctx.cu_seqlens, H, G, N, dv, write=dt, skip=self.skip,
+                               chunk_plan=K.step_chunk_plan(ctx, N))
         y = K.group_gated_norm(o, proj[:, :inner], self.norm_weight, inner // self.norm_groups, self.eps, "silu",
                                gate_first=True, out_scale=self.out_scale)
         return K.linear(y, self.w_o, partial_ok=True)

@@ -382,6 +382,14 @@ def test_recurrence_kernel(delta, heads, qk_heads, dim, vdim):
         assert float((out.cpu().double().view(n, heads, vdim) - want).abs().max()) <= 3e-5 * scale, f"per_token={per_token}"
         assert float((state.cpu().double() - want_state).abs().max()) <= 3e-5 * float(want_state.abs().max())
         assert torch.equal(state[1].cpu(), state0[1]) and torch.equal(state[4].cpu(), state0[4])    # other slots untouched
+        if K.recurrence_chunks_possible(dim, delta):       # the same by chunks of tokens side by side
+            state = state0.cuda().clone()
+            out = K.recurrence_steps(wc[:, :qk_heads * dim], wc[:, qk_heads * dim + 3:], v.cuda(), (gg if per_token else gg[0]).contiguous().cuda(),
+                                     state, sl, cu, heads, qk_heads, dim, vdim, write=wgt.cuda() if with_w else None,
+                                     skip=skip.cuda() if with_skip else None, chunk_plan=K.recurrence_chunk_plan(lens, "cuda"))
+            assert float((out.cpu().double().view(n, heads, vdim) - want).abs().max()) <= 3e-5 * scale, f"chunks, per_token={per_token}"
+            assert float((state.cpu().double() - want_state).abs().max()) <= 3e-5 * float(want_state.abs().max())
+            assert torch.equal(state[1].cpu(), state0[1]) and torch.equal(state[4].cpu(), state0[4])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
@@ -448,19 +456,24 @@ def test_gates_heads_and_norms_around_the_recurrence(dtype):
     wantu = xv / torch.sqrt((xv * xv).sum(-1, keepdim=True) + 1e-6) * torch.tensor([0.5, 2.0, 2.0, 2.0], dtype=torch.float64)[None, :, None]
     assert float((y.cpu().double()[:, :4 * d].view(n, 4, d) - wantu).abs().max()) < 1e-6
     assert torch.equal(y.cpu()[:, 4 * d:], x[:, 4 * d:])
-    o = torch.randn(n, 24, generator=gen)
-    weight = 1 + 0.3 * torch.randn(8, generator=gen)
-    gate = proj[:, 40:64]
-    for group, first, act, wt in ((8, False, "silu", weight), (12, True, "silu", None), (24, False, "sigmoid", weight), (4, True, "sigmoid", weight)):
-        a = torch.nn.functional.silu(gate.double()) if act == "silu" else torch.sigmoid(gate.double())
-        z = o.double() * a if first else o.double()
-        z = (z.view(n, -1, group) / torch.sqrt((z.view(n, -1, group) ** 2).mean(-1, keepdim=True) + 1e-3)).view(n, 24)
-        if wt is not None:
-            z = z * wt.double().repeat(3)
-        z = (z if first else z * a) * 0.7
-        got = K.group_gated_norm(o.cuda(), proj.cuda()[:, 40:64], None if wt is None else wt.cuda(), group, 1e-3, act, gate_first=first, out_scale=0.7)
-        tol = 1e-5 if dtype == torch.float32 else 1e-2
-        assert float((got.cpu().double() - z).abs().max()) <= tol * max(1.0, float(z.abs().max())), (group, first, act)
+    wide = (torch.randn(n, 610, generator=gen) * 2).to(dtype)
+    for width, weight_len, cases in ((24, 8, ((8, False, "silu", True), (12, True, "silu", False), (24, False, "sigmoid", True), (4, True, "sigmoid", True))),
+                                     (600, 300, ((300, True, "silu", True), (600, False, "silu", False)))):      # wide groups take a block each
+        o = torch.randn(n, width, generator=gen)
+        weight = 1 + 0.3 * torch.randn(weight_len, generator=gen)
+        src = proj if width == 24 else wide
+        gate = src[:, 10:10 + width]
+        for group, first, act, weighted in cases:
+            a = torch.nn.functional.silu(gate.double()) if act == "silu" else torch.sigmoid(gate.double())
+            z = o.double() * a if first else o.double()
+            z = (z.view(n, -1, group) / torch.sqrt((z.view(n, -1, group) ** 2).mean(-1, keepdim=True) + 1e-3)).view(n, width)
+            if weighted:
+                z = z * weight.double().repeat(width // weight_len)
+            z = (z if first else z * a) * 0.7
+            got = K.group_gated_norm(o.cuda(), src.cuda()[:, 10:10 + width], weight.cuda() if weighted else None, group, 1e-3, act,
+                                     gate_first=first, out_scale=0.7)
+            tol = 1e-5 if dtype == torch.float32 else 1e-2
+            assert float((got.cpu().double() - z).abs().max()) <= tol * max(1.0, float(z.abs().max())), (group, first, act)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
