@@ -422,7 +422,7 @@ recurrence_apply_kernel(float* __restrict__ out, const float* __restrict__ scrat
   for (int a = 0; a < 4; ++a) {
     const int i = i0 + a;
     if (i >= n) continue;
-    const float w = cum[(long long)(b0 + i) * heads + h];
+    const float w = cum ? cum[(long long)(b0 + i) * heads + h] : 1.f;
     float* dst = out + (long long)(b0 + i) * heads * vdim + h * vdim + c0 + c;
 #pragma unroll
     for (int b = 0; b < 4; ++b)
@@ -454,6 +454,287 @@ extern "C" int jv_recurrence_chunks(float* out, const float* q, long long ldq, c
                      state, cum, slot_ids, req_chunks, work, cu_seqlens, heads, dim, vdim);
   hipLaunchKernelGGL(recurrence_apply_kernel, dim3(chunks, heads, slices), dim3(256), lds_apply, s, out, scratch, cum, q,
                      ldq, work, cu_seqlens, heads, qk_heads, dim, vdim);
+  return JV_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------- the delta rule by chunks
+// Inside a chunk (c_i as above, G_i = exp(c_i), beta_i the write strength, S0 the state before it) the updates
+//     u_i = beta_i (v_i - (g_i S_(i-1))^T k_i),   S_i = g_i S_(i-1) + k_i u_i^T
+// obey  u_i = beta_i (v_i - G_i S0^T k_i - sum_{j<i} A_ij u_j),  A_ij = exp(c_i - c_j) (k_i . k_j), so with the lower
+// triangular T = (I + diag(beta) A)^-1 diag(beta):
+//     U = Wv - Wk S0,             Wv = T V,  Wk = T diag(G) K
+//     O = Qt S0 + (B T) V,        B_ij = exp(c_i - c_j) (q_i . k_j) (j <= i),  Qt = diag(G) Q - (B T) diag(G) K
+//     S_end = G_(n-1) S0 + Kd^T U,   Kd_j = exp(c_(n-1) - c_j) k_j
+// Three launches: `local` makes T, Wk, Kd, Qt, Wv and the chunk-local outputs (B T) V for all chunks side by side;
+// `scan` walks a request's chunks in order with a slice of S in LDS (two small products a chunk) and leaves the state
+// before every chunk in scratch; the plain recurrence's `apply` adds Qt S_before.
+// grid (chunks, heads)
+__global__ void __launch_bounds__(256)
+delta_local_kernel(float* __restrict__ out, float* __restrict__ wk_out, float* __restrict__ kd_out,
+                   float* __restrict__ wv_out, float* __restrict__ qt_out, float* __restrict__ cum,
+                   const float* __restrict__ q, long long ldq, const float* __restrict__ k, long long ldk,
+                   const float* __restrict__ v, long long ldv, const float* __restrict__ g, int g_stride,
+                   const float* __restrict__ wgt, const int* __restrict__ work, const int* __restrict__ cu_seqlens,
+                   int heads, int qk_heads, int dim, int vdim) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int ch = blockIdx.x, h = blockIdx.y;
+  const int r = work[2 * ch], b0 = work[2 * ch + 1];
+  const int n = min(RC_LC, cu_seqlens[r + 1] - b0);
+  const int hk = h / (heads / qk_heads);
+  const int dq = dim + RC_PAD, lm = RC_LC + 1;
+  float* qs = lds;                       // [LC][dq]
+  float* ks = qs + RC_LC * dq;           // [LC][dq]
+  float* ma = ks + RC_LC * dq;           // [LC][LC + 1]: A, later B T
+  float* mb = ma + RC_LC * lm;           // [LC][LC + 1]: B
+  float* mt = mb + RC_LC * lm;           // [LC][LC + 1]: T
+  float* vs = mt + RC_LC * lm;           // [LC][LV]
+  float* cl = vs + RC_LC * RC_LV;        // [LC] cumulative log decay
+  float* bs = cl + RC_LC;                // [LC] beta
+  float* gs = bs + RC_LC;                // [LC] exp(cl)
+  const int tid = threadIdx.x;
+  if (tid < RC_LC) {
+    float lg = 0.f, w = 0.f;
+    if (tid < n) {
+      lg = logf(fmaxf(g[(long long)(b0 + tid) * g_stride + h], 1e-38f));
+      w = wgt ? wgt[(long long)(b0 + tid) * heads + h] : 1.f;
+    }
+#pragma unroll
+    for (int o = 1; o < RC_LC; o <<= 1) {
+      const float up = __shfl_up(lg, o, JV_WAVE);
+      if (tid >= o) lg += up;
+    }
+    cl[tid] = lg;
+    bs[tid] = w;
+    gs[tid] = expf(lg);
+    if (tid < n) cum[(long long)(b0 + tid) * heads + h] = expf(lg);
+  }
+  for (int i = tid; i < RC_LC * dq; i += 256) {
+    const int j = i / dq, d = i - j * dq;
+    float qv = 0.f, kv = 0.f;
+    if (j < n && d < dim) {
+      qv = q[(long long)(b0 + j) * ldq + hk * dim + d];
+      kv = k[(long long)(b0 + j) * ldk + hk * dim + d];
+    }
+    qs[i] = qv;
+    ks[i] = kv;
+  }
+  __syncthreads();
+  {  // A (below the diagonal) and B (with the diagonal): thread (i, 4 consecutive j)
+    const int i = tid >> 3, j0 = (tid & 7) * 4;
+    float da[4] = {0.f, 0.f, 0.f, 0.f}, db[4] = {0.f, 0.f, 0.f, 0.f};
+    if (j0 <= i) {
+      for (int d = 0; d < dim; ++d) {
+        const float kv = ks[i * dq + d], qv = qs[i * dq + d];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float kj = ks[(j0 + u) * dq + d];
+          da[u] = fmaf(kv, kj, da[u]);
+          db[u] = fmaf(qv, kj, db[u]);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u;
+      const float f = (j <= i && i < n) ? expf(cl[i] - cl[j]) : 0.f;
+      ma[i * lm + j] = j < i ? da[u] * f : 0.f;
+      mb[i * lm + j] = db[u] * f;
+    }
+  }
+  __syncthreads();
+  if (tid < RC_LC) {   // column tid of T: t_i = beta_i (e_i - sum_{j<i} A_ij t_j); a column depends on itself only
+    const int c = tid;
+    for (int i = 0; i < RC_LC; ++i) {
+      float acc = i == c ? 1.f : 0.f;
+      for (int j = c; j < i; ++j) acc = fmaf(-ma[i * lm + j], mt[j * lm + c], acc);
+      mt[i * lm + c] = i < c ? 0.f : bs[i] * acc;
+    }
+  }
+  // Kd from the plain keys, meanwhile
+  float* wk_c = wk_out + ((long long)ch * heads + h) * RC_LC * dim;
+  float* kd_c = kd_out + ((long long)ch * heads + h) * RC_LC * dim;
+  for (int e = tid; e < RC_LC * dim; e += 256) {
+    const int i = e / dim, d = e - i * dim;
+    kd_c[e] = i < n ? ks[i * dq + d] * expf(cl[n - 1] - cl[i]) : 0.f;
+  }
+  __syncthreads();
+  {  // B T into A's place; keys times G in place
+    const int i = tid >> 3, j0 = (tid & 7) * 4;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int m = j0; m <= i; ++m) {
+      const float b = mb[i * lm + m];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc[u] = fmaf(b, mt[m * lm + j0 + u], acc[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) ma[i * lm + j0 + u] = acc[u];
+    for (int e = tid; e < RC_LC * dq; e += 256) ks[e] *= gs[e / dq];
+  }
+  __syncthreads();
+  // Wk = T (G K);  Qt = G Q - (B T)(G K)
+  for (int e = tid; e < RC_LC * dim; e += 256) {
+    const int i = e / dim, d = e - i * dim;
+    float a = 0.f, b = 0.f;
+    for (int j = 0; j <= i; ++j) {
+      const float kv = ks[j * dq + d];
+      a = fmaf(mt[i * lm + j], kv, a);
+      b = fmaf(ma[i * lm + j], kv, b);
+    }
+    wk_c[e] = a;
+    if (i < n) qt_out[((long long)(b0 + i) * heads + h) * dim + d] = gs[i] * qs[i * dq + d] - b;
+  }
+  // Wv = T V and the chunk's own outputs (B T) V, a slice of columns at a time
+  float* wv_c = wv_out + ((long long)ch * heads + h) * RC_LC * vdim;
+  for (int c0 = 0; c0 < vdim; c0 += RC_LV) {
+    const int ncols = min(RC_LV, vdim - c0);
+    __syncthreads();
+    for (int i = tid; i < RC_LC * RC_LV; i += 256) {
+      const int j = i / RC_LV, c = i % RC_LV;
+      vs[i] = (j < n && c < ncols) ? v[(long long)(b0 + j) * ldv + h * vdim + c0 + c] : 0.f;
+    }
+    __syncthreads();
+    for (int e = tid; e < RC_LC * (RC_LV / 4); e += 256) {
+      const int i = e / (RC_LV / 4), c = (e % (RC_LV / 4)) * 4;
+      if (c >= ncols) continue;
+      float4 wv = {0.f, 0.f, 0.f, 0.f}, o = {0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j <= i; ++j) {
+        const float t = mt[i * lm + j], a = ma[i * lm + j];
+        const float4 x = *(const float4*)(vs + j * RC_LV + c);
+        wv.x = fmaf(t, x.x, wv.x); wv.y = fmaf(t, x.y, wv.y); wv.z = fmaf(t, x.z, wv.z); wv.w = fmaf(t, x.w, wv.w);
+        o.x = fmaf(a, x.x, o.x); o.y = fmaf(a, x.y, o.y); o.z = fmaf(a, x.z, o.z); o.w = fmaf(a, x.w, o.w);
+      }
+      float* wd = wv_c + (long long)i * vdim + c0 + c;
+      const float wvv[4] = {wv.x, wv.y, wv.z, wv.w}, ov[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (c + u < ncols) {
+          wd[u] = wvv[u];
+          if (i < n) out[(long long)(b0 + i) * heads * vdim + h * vdim + c0 + c + u] = ov[u];
+        }
+    }
+  }
+}
+
+#define RC_DS 32        // columns of the state a block of the delta scan keeps
+// grid (requests, heads, column slices of RC_DS)
+__global__ void __launch_bounds__(256)
+delta_scan_kernel(float* __restrict__ sb, float* __restrict__ state, const float* __restrict__ wk_in,
+                  const float* __restrict__ kd_in, const float* __restrict__ wv_in, const float* __restrict__ cum,
+                  const int* __restrict__ slot_ids, const int* __restrict__ req_chunks, const int* __restrict__ work,
+                  const int* __restrict__ cu_seqlens, int heads, int dim, int vdim) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int r = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * RC_DS;
+  const int first = req_chunks[r], last = req_chunks[r + 1];
+  if (last <= first) return;
+  const int dq = dim + RC_PAD, lu = RC_DS + 4;
+  float* ss = lds;                       // [dim][RC_DS]
+  float* wk = ss + dim * RC_DS;          // [LC][dq]
+  float* kd = wk + RC_LC * dq;           // [LC][dq]
+  float* us = kd + RC_LC * dq;           // [LC][RC_DS + 4]: Wv, then U
+  const int tid = threadIdx.x;
+  const int ncols = min(RC_DS, vdim - c0);
+  float* S = state + ((long long)slot_ids[r] * heads + h) * dim * vdim + c0;
+  for (int e = tid; e < dim * RC_DS; e += 256) {
+    const int d = e / RC_DS, c = e % RC_DS;
+    ss[e] = c < ncols ? S[(long long)d * vdim + c] : 0.f;
+  }
+  const int end = cu_seqlens[r + 1];
+  for (int ch = first; ch < last; ++ch) {
+    const float* wk_c = wk_in + ((long long)ch * heads + h) * RC_LC * dim;
+    const float* kd_c = kd_in + ((long long)ch * heads + h) * RC_LC * dim;
+    const float* wv_c = wv_in + ((long long)ch * heads + h) * RC_LC * vdim + c0;
+    float* sb_c = sb + ((long long)ch * heads + h) * dim * vdim + c0;
+    __syncthreads();       // the turn before has read wk, kd, us and written ss
+    for (int e = tid; e < RC_LC * dim; e += 256) {
+      const int i = e / dim, d = e - i * dim;
+      wk[i * dq + d] = wk_c[e];
+      kd[i * dq + d] = kd_c[e];
+    }
+    for (int e = tid; e < RC_LC * RC_DS; e += 256) {
+      const int i = e / RC_DS, c = e % RC_DS;
+      us[i * lu + c] = c < ncols ? wv_c[(long long)i * vdim + c] : 0.f;
+    }
+    for (int e = tid; e < dim * RC_DS; e += 256) {       // the state before this chunk, for `apply`
+      const int d = e / RC_DS, c = e % RC_DS;
+      if (c < ncols) sb_c[(long long)d * vdim + c] = ss[e];
+    }
+    __syncthreads();
+    {  // U = Wv - Wk S: thread (token i, 4 columns)
+      const int i = tid >> 3, c = (tid & 7) * 4;
+      float4 p = {0.f, 0.f, 0.f, 0.f};
+      for (int d = 0; d < dim; ++d) {
+        const float w = wk[i * dq + d];
+        const float4 x = *(const float4*)(ss + d * RC_DS + c);
+        p.x = fmaf(w, x.x, p.x); p.y = fmaf(w, x.y, p.y); p.z = fmaf(w, x.z, p.z); p.w = fmaf(w, x.w, p.w);
+      }
+      float4* u = (float4*)(us + i * lu + c);
+      float4 w4 = *u;
+      w4.x -= p.x; w4.y -= p.y; w4.z -= p.z; w4.w -= p.w;
+      *u = w4;
+    }
+    __syncthreads();
+    const int b0 = work[2 * ch + 1];
+    const int n = min(RC_LC, end - b0);
+    const float gn = cum[(long long)(b0 + n - 1) * heads + h];
+    for (int e = tid; e < (dim / 4) * (RC_DS / 4); e += 256) {      // S = G S + Kd^T U: tiles of 4 x 4
+      const int d0 = (e / (RC_DS / 4)) * 4, c = (e % (RC_DS / 4)) * 4;
+      float acc[4][4];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const float4 x = *(const float4*)(ss + (d0 + a) * RC_DS + c);
+        acc[a][0] = gn * x.x; acc[a][1] = gn * x.y; acc[a][2] = gn * x.z; acc[a][3] = gn * x.w;
+      }
+      for (int j = 0; j < n; ++j) {
+        const float4 kv = *(const float4*)(kd + j * dq + d0);
+        const float4 uv = *(const float4*)(us + j * lu + c);
+        const float kk[4] = {kv.x, kv.y, kv.z, kv.w}, uu[4] = {uv.x, uv.y, uv.z, uv.w};
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int b = 0; b < 4; ++b) acc[a][b] = fmaf(kk[a], uu[b], acc[a][b]);
+      }
+#pragma unroll
+      for (int a = 0; a < 4; ++a) *(float4*)(ss + (d0 + a) * RC_DS + c) = float4{acc[a][0], acc[a][1], acc[a][2], acc[a][3]};
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < dim * RC_DS; e += 256) {
+    const int d = e / RC_DS, c = e % RC_DS;
+    if (c < ncols) S[(long long)d * vdim + c] = ss[e];
+  }
+}
+
+// scratch: floats for chunks * heads * (2 * LC * dim + LC * vdim + dim * vdim) + tokens * heads * dim; cum: tokens * heads
+extern "C" long long jv_delta_chunks_scratch_floats(int chunks, int tokens, int heads, int dim, int vdim) {
+  return (long long)chunks * heads * (2LL * RC_LC * dim + (long long)RC_LC * vdim + (long long)dim * vdim) +
+         (long long)tokens * heads * dim;
+}
+
+extern "C" int jv_delta_chunks(float* out, const float* q, long long ldq, const float* k, long long ldk,
+                               const float* v, long long ldv, const float* g, int g_stride, const float* wgt,
+                               float* state, const int* slot_ids, const int* cu_seqlens, int n_requests, int n_tokens,
+                               int heads, int qk_heads, int dim, int vdim, int chunks, const int* work,
+                               const int* req_chunks, float* scratch, float* cum, void* stream) {
+  if (n_requests <= 0 || heads <= 0 || chunks <= 0) return 0;
+  if (dim <= 0 || dim > 128 || dim % 4 || vdim <= 0 || heads > 65535 || qk_heads <= 0 || heads % qk_heads || !work ||
+      !req_chunks || !scratch || !cum)
+    return (int)hipErrorInvalidValue;
+  hipStream_t s = (hipStream_t)stream;
+  const long long per = (long long)chunks * heads;
+  float* wk = scratch;
+  float* kd = wk + per * RC_LC * dim;
+  float* wv = kd + per * RC_LC * dim;
+  float* sb = wv + per * RC_LC * vdim;
+  float* qt = sb + per * dim * vdim;
+  const size_t lds_local = (2 * RC_LC * (dim + RC_PAD) + 3 * RC_LC * (RC_LC + 1) + RC_LC * RC_LV + 3 * RC_LC) * sizeof(float);
+  const size_t lds_scan = ((size_t)dim * RC_DS + 2 * RC_LC * (dim + RC_PAD) + RC_LC * (RC_DS + 4)) * sizeof(float);
+  const size_t lds_apply = (RC_LC * (dim + 1) + 32 * RC_LV) * sizeof(float);
+  hipLaunchKernelGGL(delta_local_kernel, dim3(chunks, heads), dim3(256), lds_local, s, out, wk, kd, wv, qt, cum, q, ldq,
+                     k, ldk, v, ldv, g, g_stride, wgt, work, cu_seqlens, heads, qk_heads, dim, vdim);
+  hipLaunchKernelGGL(delta_scan_kernel, dim3(n_requests, heads, (vdim + RC_DS - 1) / RC_DS), dim3(256), lds_scan, s, sb,
+                     state, wk, kd, wv, cum, slot_ids, req_chunks, work, cu_seqlens, heads, dim, vdim);
+  hipLaunchKernelGGL(recurrence_apply_kernel, dim3(chunks, heads, (vdim + RC_LV - 1) / RC_LV), dim3(256), lds_apply, s,
+                     out, sb, (const float*)nullptr, qt, (long long)heads * dim, work, cu_seqlens, heads, heads, dim, vdim);
   return JV_LAUNCH_CHECK();
 }
 

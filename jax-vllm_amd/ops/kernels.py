@@ -1167,7 +1167,7 @@ def recurrence_steps(q, k, v, decay, state, slot_ids, cu_seqlens, heads: int, qk
     ``q``, ``k``: float views [n, qk_heads * dim] (unit column stride; head h reads q/k head h // (heads // qk_heads)),
     ``v`` a float view [n, heads * vdim]; ``decay`` g: float [n, heads] or [heads] (constant per head); ``write`` w:
     float [n, heads] or None (1); ``skip``: float [heads] or None.  ``chunk_plan`` (``recurrence_chunk_plan`` of the
-    step's token counts; not for ``delta``): the kernels that take a request's tokens a chunk at a time, chunks side
+    step's token counts): the kernels that take a request's tokens a chunk at a time, chunks side
     by side, instead of one by one (the same numbers in another order of operations)."""
     _dev(decay, write, skip, state, slot_ids, cu_seqlens)
     n = v.shape[0]
@@ -1192,12 +1192,24 @@ def recurrence_steps(q, k, v, decay, state, slot_ids, cu_seqlens, heads: int, qk
         return out
     if chunk_plan is not None:
         work, first, chunks = chunk_plan
-        _need(recurrence_chunks_possible(dim, delta), "the kernels by chunks take key sizes that are multiples of 4, at most 128, and no delta rule")
+        _need(recurrence_chunks_possible(dim, delta), "the kernels by chunks take key sizes that are multiples of 4, at most 128")
         _dev(work, first)
         _i32(work, "work", 2 * chunks)
         _i32(first, "first chunks", r + 1)
-        scratch = torch.empty(chunks * heads * dim * vdim, dtype=torch.float32, device=v.device)
         cum = torch.empty(n * heads, dtype=torch.float32, device=v.device)
+        if delta:
+            _need(skip is None, "the delta rule by chunks has no skip term")
+            lib = library.core()
+            lib.jv_delta_chunks_scratch_floats.restype = c_longlong
+            scratch = torch.empty(lib.jv_delta_chunks_scratch_floats(c_int(chunks), c_int(n), c_int(heads), c_int(dim), c_int(vdim)),
+                                  dtype=torch.float32, device=v.device)
+            _check(lib.jv_delta_chunks(
+                _ptr(out), _ptr(q), c_longlong(q.stride(0)), _ptr(k), c_longlong(k.stride(0)), _ptr(v), c_longlong(v.stride(0)),
+                _ptr(decay), c_int(heads if decay.dim() == 2 else 0), _ptr(write), _ptr(state), _ptr(slot_ids), _ptr(cu_seqlens),
+                c_int(r), c_int(n), c_int(heads), c_int(qk_heads), c_int(dim), c_int(vdim), c_int(chunks), _ptr(work), _ptr(first),
+                _ptr(scratch), _ptr(cum), _stream()), "delta_chunks")
+            return out
+        scratch = torch.empty(chunks * heads * dim * vdim, dtype=torch.float32, device=v.device)
         _check(library.core().jv_recurrence_chunks(
             _ptr(out), _ptr(q), c_longlong(q.stride(0)), _ptr(k), c_longlong(k.stride(0)), _ptr(v), c_longlong(v.stride(0)),
             _ptr(decay), c_int(heads if decay.dim() == 2 else 0), _ptr(write), _ptr(skip), _ptr(state), _ptr(slot_ids),
@@ -1220,8 +1232,9 @@ def recurrence_chunk_tokens() -> int:
 
 
 def recurrence_chunks_possible(dim: int, delta: bool = False) -> bool:
-    """The kernels by chunks keep a chunk's keys in LDS in 16-byte pieces; the delta rule runs token by token."""
-    return not delta and dim % 4 == 0 and dim <= library.core().jv_recurrence_chunk_max_dim()
+    """The kernels by chunks (of the plain recurrence and of the delta rule alike) keep a chunk's keys in LDS in
+    16-byte pieces."""
+    return dim % 4 == 0 and dim <= library.core().jv_recurrence_chunk_max_dim()
 
 
 def recurrence_chunk_plan(q_lens, device):

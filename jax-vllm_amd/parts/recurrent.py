@@ -194,7 +194,7 @@ class GatedDeltaMixer:
         q, k, v = qkv[:, :qk], qkv[:, qk:2 * qk], qkv[:, 2 * qk:]
         K.head_unit_norm(qkv, 2 * self.qk_heads, d, self.unit_eps, 1.0, first_heads=self.qk_heads, first_scale=d ** -0.5)
         o = K.recurrence_steps(q, k, v, g, mem.states["S"], ctx.slot_ids, ctx.cu_seqlens, H, self.qk_heads, d, dv,
-                               write=beta, delta=True)
+                               write=beta, delta=True, chunk_plan=K.step_chunk_plan(ctx, d, delta=True))
         y = K.group_gated_norm(o, proj[:, gate_at:gate_at + inner], self.norm_weight, dv, self.eps, "silu",
                                out_scale=self.out_scale)
         return K.linear(y, self.w_o, partial_ok=True)

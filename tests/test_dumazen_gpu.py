@@ -386,7 +386,10 @@ def test_recurrence_kernel(delta, heads, qk_heads, dim, vdim):
             state = state0.cuda().clone()
             out = K.recurrence_steps(wc[:, :qk_heads * dim], wc[:, qk_heads * dim + 3:], v.cuda(), (gg if per_token else gg[0]).contiguous().cuda(),
                                      state, sl, cu, heads, qk_heads, dim, vdim, write=wgt.cuda() if with_w else None,
-                                     skip=skip.cuda() if with_skip else None, chunk_plan=K.recurrence_chunk_plan(lens, "cuda"))
+                                     skip=skip.cuda() if with_skip and not delta else None, delta=delta,
+                                     chunk_plan=K.recurrence_chunk_plan(lens, "cuda"))
+            if delta and with_skip:
+                out = out + (skip.cuda()[None, :, None] * v.cuda().view(n, heads, vdim)).view(n, -1)
             assert float((out.cpu().double().view(n, heads, vdim) - want).abs().max()) <= 3e-5 * scale, f"chunks, per_token={per_token}"
             assert float((state.cpu().double() - want_state).abs().max()) <= 3e-5 * float(want_state.abs().max())
             assert torch.equal(state[1].cpu(), state0[1]) and torch.equal(state[4].cpu(), state0[4])
