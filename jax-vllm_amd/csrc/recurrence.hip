@@ -616,6 +616,9 @@ delta_local_kernel(float* __restrict__ out, float* __restrict__ wk_out, float* _
 }
 
 #define RC_DS 32        // columns of the state a block of the delta scan keeps
+// A barrier that waits for the block's LDS traffic only: loads from global memory that were asked for a turn ahead stay
+// in flight across it (`__syncthreads` would wait for them too).
+__device__ __forceinline__ void rc_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 // grid (requests, heads, column slices of RC_DS)
 __global__ void __launch_bounds__(256)
 delta_scan_kernel(float* __restrict__ sb, float* __restrict__ state, const float* __restrict__ wk_in,
@@ -639,26 +642,52 @@ delta_scan_kernel(float* __restrict__ sb, float* __restrict__ state, const float
     ss[e] = c < ncols ? S[(long long)d * vdim + c] : 0.f;
   }
   const int end = cu_seqlens[r + 1];
-  for (int ch = first; ch < last; ++ch) {
+  // a chunk's Wk, Kd and Wv travel through registers: they are asked for a turn ahead, while the turn before computes
+  constexpr int RK = RC_LC * 128 / 256, RU = RC_LC * RC_DS / 256;
+  float rw[RK], rk[RK], ru[RU];
+  int at[RK];            // where a thread's pieces of Wk and Kd go in LDS (-1: beyond the chunk)
+#pragma unroll
+  for (int u = 0; u < RK; ++u) {
+    const int e = tid + u * 256;
+    at[u] = e < RC_LC * dim ? (e / dim) * dq + e % dim : -1;
+  }
+  auto fetch = [&](int ch) {
     const float* wk_c = wk_in + ((long long)ch * heads + h) * RC_LC * dim;
     const float* kd_c = kd_in + ((long long)ch * heads + h) * RC_LC * dim;
     const float* wv_c = wv_in + ((long long)ch * heads + h) * RC_LC * vdim + c0;
-    float* sb_c = sb + ((long long)ch * heads + h) * dim * vdim + c0;
-    __syncthreads();       // the turn before has read wk, kd, us and written ss
-    for (int e = tid; e < RC_LC * dim; e += 256) {
-      const int i = e / dim, d = e - i * dim;
-      wk[i * dq + d] = wk_c[e];
-      kd[i * dq + d] = kd_c[e];
+#pragma unroll
+    for (int u = 0; u < RK; ++u) {
+      const int e = min(tid + u * 256, RC_LC * dim - 1);       // a piece beyond the chunk reads its last element, unused
+      rw[u] = wk_c[e];
+      rk[u] = kd_c[e];
     }
-    for (int e = tid; e < RC_LC * RC_DS; e += 256) {
-      const int i = e / RC_DS, c = e % RC_DS;
-      us[i * lu + c] = c < ncols ? wv_c[(long long)i * vdim + c] : 0.f;
+#pragma unroll
+    for (int u = 0; u < RU; ++u) {
+      const int e = tid + u * 256, i = e / RC_DS, c = e % RC_DS;
+      ru[u] = wv_c[(long long)i * vdim + min(c, ncols - 1)];
+    }
+  };
+  fetch(first);
+  for (int ch = first; ch < last; ++ch) {
+    float* sb_c = sb + ((long long)ch * heads + h) * dim * vdim + c0;
+    rc_lds_barrier();      // the turn before has read wk, kd, us and written ss
+#pragma unroll
+    for (int u = 0; u < RK; ++u)
+      if (at[u] >= 0) {
+        wk[at[u]] = rw[u];
+        kd[at[u]] = rk[u];
+      }
+#pragma unroll
+    for (int u = 0; u < RU; ++u) {
+      const int e = tid + u * 256, i = e / RC_DS, c = e % RC_DS;
+      us[i * lu + c] = c < ncols ? ru[u] : 0.f;
     }
     for (int e = tid; e < dim * RC_DS; e += 256) {       // the state before this chunk, for `apply`
       const int d = e / RC_DS, c = e % RC_DS;
       if (c < ncols) sb_c[(long long)d * vdim + c] = ss[e];
     }
-    __syncthreads();
+    rc_lds_barrier();
+    fetch(min(ch + 1, last - 1));       // never conditional: the last turn asks for its own chunk again
     {  // U = Wv - Wk S: thread (token i, 4 columns)
       const int i = tid >> 3, c = (tid & 7) * 4;
       float4 p = {0.f, 0.f, 0.f, 0.f};
@@ -672,7 +701,7 @@ delta_scan_kernel(float* __restrict__ sb, float* __restrict__ state, const float
       w4.x -= p.x; w4.y -= p.y; w4.z -= p.z; w4.w -= p.w;
       *u = w4;
     }
-    __syncthreads();
+    rc_lds_barrier();
     const int b0 = work[2 * ch + 1];
     const int n = min(RC_LC, end - b0);
     const float gn = cum[(long long)(b0 + n - 1) * heads + h];
