@@ -115,6 +115,31 @@ heads_to_f32_kernel(float* __restrict__ out, const T* __restrict__ proj, long lo
   out[e] = x * scale;
 }
 
+// The same for q, k and v of one mixer at once: proj rows [q: heads * d | k: heads * d | v: heads * dv | ...] become float
+// rows [q | k | v]; q and k turn by position, k is multiplied by k_scale, v is copied.
+template <typename T>
+__global__ void __launch_bounds__(256)
+qkv_to_f32_kernel(float* __restrict__ out, const T* __restrict__ proj, long long ld, int n, int heads, int d, int dv,
+                  int rot_dims, const float* __restrict__ cos_sin, float k_scale) {
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+  const int qk = heads * d, width = 2 * qk + heads * dv;
+  if (e >= (long long)n * width) return;
+  const int t = (int)(e / width), c = (int)(e % width);
+  const T* row = proj + (long long)t * ld;
+  float x = to_f32(row[c]);
+  if (c < 2 * qk) {
+    const int i = c % d;
+    if (i < rot_dims) {
+      const int half = rot_dims / 2, j = i < half ? i : i - half;
+      const float cs = cos_sin[(long long)t * rot_dims + j], sn = cos_sin[(long long)t * rot_dims + half + j];
+      const float other = to_f32(row[i < half ? c + half : c - half]);
+      x = i < half ? x * cs - other * sn : x * cs + other * sn;
+    }
+    if (c >= qk) x *= k_scale;
+  }
+  out[e] = x;
+}
+
 // x [n][ld] float, in place on the first `heads` runs of d columns of every row: x / sqrt(sum(x^2) + eps) * scale,
 // scale = scale_a for the first `heads_a` heads of a row and scale_b for the others; one wave a head
 __global__ void __launch_bounds__(256)
@@ -890,6 +915,16 @@ extern "C" int jv_recurrence_steps(float* out, const float* q, long long ldq, co
     hipLaunchKernelGGL(heads_to_f32_kernel<T>, dim3((unsigned)(((long long)n * heads * d + 255) / 256)),       \
                        dim3(256), 0, (hipStream_t)stream, out, (const T*)proj, ld, off, n, heads, d, rot_dims, \
                        cos_sin, scale);                                                                        \
+    return JV_LAUNCH_CHECK();                                                                                  \
+  }                                                                                                            \
+  extern "C" int jv_qkv_to_f32_##SUF(float* out, const void* proj, long long ld, int n, int heads, int d,      \
+                                     int dv, int rot_dims, const float* cos_sin, float k_scale, void* stream) { \
+    if (n <= 0 || heads <= 0 || d <= 0 || dv <= 0) return 0;                                                   \
+    if (rot_dims < 0 || rot_dims > d || rot_dims % 2 || (rot_dims && !cos_sin)) return (int)hipErrorInvalidValue; \
+    const long long total = (long long)n * (2LL * heads * d + (long long)heads * dv);                          \
+    hipLaunchKernelGGL(qkv_to_f32_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,              \
+                       (hipStream_t)stream, out, (const T*)proj, ld, n, heads, d, dv, rot_dims, cos_sin,       \
+                       k_scale);                                                                               \
     return JV_LAUNCH_CHECK();                                                                                  \
   }                                                                                                            \
   extern "C" int jv_group_gated_norm_##SUF(void* out, const float* o, const void* gate, long long g_stride,    \

@@ -5,7 +5,7 @@
 
 // ---------------------------------------------------------------- post-norm + residual add + next pre-norm
 // Row r = rows ? rows[i] : i.
-//   v   = (y ? y[r] : 0) + parts[0][r] + parts[1][r] + ...       (the sublayer's output; parts added in order)
+//   v   = (y ? y[r] : 0) + parts[0][r] + parts[1][r] + ... (+ bias)   (the sublayer's output; parts added in order)
 //   x   = h[r] + v * rsqrt(mean(v^2) + eps) * wb                 (float)
 //   if (!rows) h[r] = x
 //   if (out)   out[i] = T( x * rsqrt(mean(x^2) + eps_out) * w ),   or T(x) where w is null
@@ -13,7 +13,8 @@
 template <typename T>
 __global__ void __launch_bounds__(256)
 postnorm_add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ y, const float* __restrict__ parts,
-                            int n_parts, long long part_stride, const float* __restrict__ wb,
+                            int n_parts, long long part_stride, const float* __restrict__ bias,
+                            const float* __restrict__ wb,
                             const float* __restrict__ w, T* __restrict__ out, const int* __restrict__ rows,
                             int hidden, float eps, float eps_out) {
   extern __shared__ float row[];
@@ -25,6 +26,7 @@ postnorm_add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ y, cons
   for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
     float v = y ? to_f32(y[r * hidden + c]) : 0.f;
     for (int p = 0; p < n_parts; ++p) v += parts[p * part_stride + r * hidden + c];
+    if (bias) v += bias[c];
     row[c] = v;
     ss += v * v;
   }
@@ -89,7 +91,8 @@ template <> __device__ __forceinline__ void sn_store4<float>(float* p, float4 v)
 template <typename T>
 __global__ void __launch_bounds__(256)
 postnorm_add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ y, const float* __restrict__ parts,
-                                int n_parts, long long part_stride, const float* __restrict__ wb,
+                                int n_parts, long long part_stride, const float* __restrict__ bias,
+                                const float* __restrict__ wb,
                                 const float* __restrict__ w, T* __restrict__ out, const int* __restrict__ rows,
                                 int hidden, float eps, float eps_out) {
   __shared__ float red[32];
@@ -110,6 +113,14 @@ postnorm_add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ y, 
     for (int q = 0; q < SN_V; ++q) {
       const int c = (threadIdx.x + q * 256) * 4;
       const float4 t = *(const float4*)(parts + p * part_stride + r * hidden + (c < hidden ? c : 0));
+      v[q].x += t.x; v[q].y += t.y; v[q].z += t.z; v[q].w += t.w;
+    }
+  }
+  if (bias) {
+#pragma unroll
+    for (int q = 0; q < SN_V; ++q) {
+      const int c = (threadIdx.x + q * 256) * 4;
+      const float4 t = *(const float4*)(bias + (c < hidden ? c : 0));
       v[q].x += t.x; v[q].y += t.y; v[q].z += t.z; v[q].w += t.w;
     }
   }
@@ -152,19 +163,21 @@ postnorm_add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ y, 
 
 #define DEFINE_SANDWICH(SUF, T)                                                                          \
   extern "C" int jv_postnorm_add_rmsnorm_##SUF(float* h, const void* y, const float* parts, int n_parts, \
-                                               long long part_stride, const float* wb, const float* w,   \
+                                               long long part_stride, const float* bias,               \
+                                               const float* wb, const float* w,                         \
                                                void* out, const int* rows, int n_out, int hidden,        \
                                                float eps, float eps_out, void* stream) {                 \
     if (n_out <= 0 || hidden <= 0) return 0;                                                             \
     if ((!y && n_parts <= 0) || hidden > 16384) return (int)hipErrorInvalidValue;                        \
     if (hidden % 4 == 0 && hidden <= 4 * SN_V * 256) {                                                   \
       hipLaunchKernelGGL(postnorm_add_rmsnorm_vec_kernel<T>, dim3(n_out), dim3(256), 0,                  \
-                         (hipStream_t)stream, h, (const T*)y, parts, n_parts, part_stride, wb, w,        \
+                         (hipStream_t)stream, h, (const T*)y, parts, n_parts, part_stride, bias, wb, w,  \
                          (T*)out, rows, hidden, eps, eps_out);                                           \
       return JV_LAUNCH_CHECK();                                                                          \
     }                                                                                                    \
     hipLaunchKernelGGL(postnorm_add_rmsnorm_kernel<T>, dim3(n_out), dim3(256), hidden * sizeof(float),   \
-                       (hipStream_t)stream, h, (const T*)y, parts, n_parts, part_stride, wb, w, (T*)out, \
+                       (hipStream_t)stream, h, (const T*)y, parts, n_parts, part_stride, bias, wb, w,    \
+                       (T*)out,                                                                          \
                        rows, hidden, eps, eps_out);                                                      \
     return JV_LAUNCH_CHECK();                                                                            \
   }                                                                                                      \

@@ -867,13 +867,30 @@ class PendingNorm:
     joins the residual stream: what a layer arrangement that norms the output of its sublayers hands
     to the next norm, which does both in one pass (``postnorm_add_rmsnorm``)."""
 
-    def __init__(self, y, parts, weight: torch.Tensor, eps: float):
+    def __init__(self, y, parts, weight: torch.Tensor, eps: float, bias=None):
         self.y, self.parts, self.weight, self.eps = y, parts, weight, float(eps)
+        self.bias = bias          # float [hidden] or None: a bias of the sublayer's last product, still to be added
+
+
+class BiasedOutput:
+    """What a sublayer returned (rows, a float stack, or a pair of both) whose last product's bias [hidden] is
+    still to be added: a block that norms the output lets the norm's kernel add it (``pending_norm``); anyone else
+    calls ``settled()``."""
+
+    def __init__(self, out, bias: torch.Tensor):
+        self.out, self.bias = out, bias
+
+    def settled(self):
+        rows, parts = split_sublayer_output(self.out)
+        add_bias(rows if rows is not None else parts, self.bias)
+        return self.out
 
 
 def split_sublayer_output(out):
     """(rows or None, float stack or None) of what a mixer or feed-forward returned: rows of the
     activation type, a float stack of partial results, or already a pair of both."""
+    if isinstance(out, BiasedOutput):
+        out = out.settled()
     if isinstance(out, tuple):
         return out
     if out.dim() == 3:
@@ -881,17 +898,27 @@ def split_sublayer_output(out):
     return out, None
 
 
+def pending_norm(out, weight: torch.Tensor, eps: float) -> "PendingNorm":
+    """A sublayer's output with the norm that belongs to it, for the next norm's kernel; a bias that the output still
+    owes travels along and is added there."""
+    if isinstance(out, BiasedOutput):
+        return PendingNorm(*split_sublayer_output(out.out), weight, eps, out.bias)
+    return PendingNorm(*split_sublayer_output(out), weight, eps)
+
+
 def postnorm_add_rmsnorm(h, y, parts, post_weight, eps: float, weight=None, out=None, rows=None,
-                         out_eps: float | None = None) -> None:
-    """h += norm(y + parts[0] + parts[1] + ...; post_weight) in the float residual stream, then, with
+                         out_eps: float | None = None, bias=None) -> None:
+    """h += norm(y + parts[0] + parts[1] + ... (+ bias); post_weight) in the float residual stream, then, with
     ``out``, out = norm(h; weight) (with ``out_eps``, default ``eps``) in the activation type, or h itself in that type where
     ``weight`` is None (a reader that takes the stream as it is).  With ``rows`` (int32 indices) only those
     rows are computed and h is left alone.  y is [rows of h, hidden] in the activation type or None,
     parts a float32 stack [P, rows of h, hidden] or None (any P)."""
-    _dev(h, y, parts, post_weight, weight, out, rows)
+    _dev(h, y, parts, post_weight, weight, out, rows, bias)
     _f32(h, "h")
     n, hidden = h.shape
     _f32(post_weight, "post_weight", hidden)
+    if bias is not None:       # added to the sublayer's output before its norm
+        _f32(bias, "bias", hidden)
     _need(y is not None or parts is not None, "nothing to add")
     _need(hidden <= 16384, "rows wider than 16,384 are not supported")
     if y is not None:
@@ -915,7 +942,7 @@ def postnorm_add_rmsnorm(h, y, parts, post_weight, eps: float, weight=None, out=
     kind = out.dtype if out is not None else (y.dtype if y is not None else torch.float32)
     fn = getattr(library.core(), f"jv_postnorm_add_rmsnorm_{_suffix(kind)}")
     _check(fn(_ptr(h), _ptr(y), _ptr(parts), c_int(0 if parts is None else parts.shape[0]),
-              c_longlong(0 if parts is None else parts.stride(0)), _ptr(post_weight), _ptr(weight), _ptr(out),
+              c_longlong(0 if parts is None else parts.stride(0)), _ptr(bias), _ptr(post_weight), _ptr(weight), _ptr(out),
               _ptr(rows), c_int(n_out), c_int(hidden), c_float(eps), c_float(eps if out_eps is None else out_eps), _stream()),
            "postnorm_add_rmsnorm")
 
@@ -1143,6 +1170,24 @@ def heads_to_f32(proj, off: int, heads: int, d: int, rot_dims: int = 0, cos_sin=
     fn = getattr(library.core(), f"jv_heads_to_f32_{_suffix(proj.dtype)}")
     _check(fn(_ptr(out), _ptr(proj), c_longlong(ld), c_int(off), c_int(n), c_int(heads), c_int(d), c_int(rot_dims),
               _ptr(cos_sin if rot_dims else None), c_float(scale), _stream()), "heads_to_f32")
+    return out
+
+
+def qkv_to_f32(proj, heads: int, d: int, dv: int, rot_dims: int = 0, cos_sin=None, k_scale: float = 1.0) -> torch.Tensor:
+    """Float [n, 2 * heads * d + heads * dv] = [q | k | v] of the leading columns of ``proj`` laid out the same way: the
+    first ``rot_dims`` elements of every q and k head turn by the token's angles (``rope_table``), k is multiplied by
+    ``k_scale``, v is copied: ``heads_to_f32`` for the three inputs of one mixer in one launch."""
+    _dev(proj, cos_sin)
+    n, ld = proj.shape
+    width = 2 * heads * d + heads * dv
+    _need(width <= ld, "proj rows are too short")
+    _need(rot_dims % 2 == 0 and 0 <= rot_dims <= d, "the rotated size must be even and at most the head size")
+    if rot_dims:
+        _f32(cos_sin, "cos_sin", n * rot_dims)
+    out = torch.empty((n, width), dtype=torch.float32, device=proj.device)
+    fn = getattr(library.core(), f"jv_qkv_to_f32_{_suffix(proj.dtype)}")
+    _check(fn(_ptr(out), _ptr(proj), c_longlong(ld), c_int(n), c_int(heads), c_int(d), c_int(dv), c_int(rot_dims),
+              _ptr(cos_sin if rot_dims else None), c_float(k_scale), _stream()), "qkv_to_f32")
     return out
 
 

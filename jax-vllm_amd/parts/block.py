@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import torch
 
+from ..ops import kernels as K
 from .spec import PartSpec, build_part, is_replayable, register_part
 
 
@@ -40,7 +41,8 @@ class PreNormBlock:
         x = _add_norm(self.mixer_norm, h, delta, mixer, n)
         a = mixer.forward(x, ctx, mem)
         y = _add_norm(self.feed_forward_norm, h, a, feed_forward, n)
-        return feed_forward.forward(y, ctx)
+        f = feed_forward.forward(y, ctx)
+        return f.settled() if isinstance(f, K.BiasedOutput) else f
 
 
 def _add_norm(norm, h, delta, reader, n_rows: int):
@@ -90,12 +92,12 @@ class SandwichBlock:
 
         x = self.norms[0].add_norm(h, delta)
         a = mixer.forward(x, ctx, mem)
-        pending = K.PendingNorm(*K.split_sublayer_output(a), self.norms[1].weight, self.norms[1].eps)
+        pending = K.pending_norm(a, self.norms[1].weight, self.norms[1].eps)
         if not self.has_feed_forward:
             return pending
         y = self.norms[2].add_norm(h, pending)
         f = feed_forward.forward(y, ctx)
-        return K.PendingNorm(*K.split_sublayer_output(f), self.norms[3].weight, self.norms[3].eps)
+        return K.pending_norm(f, self.norms[3].weight, self.norms[3].eps)
 
 
 class OutputNormBlock:
@@ -137,18 +139,18 @@ class OutputNormBlock:
         if not isinstance(delta, K.PendingNorm):
             raise TypeError("this arrangement follows layers that hand on a sublayer's output with its norm")
         out = torch.empty(h.shape, dtype=self.dtype, device=h.device)
-        K.postnorm_add_rmsnorm(h, delta.y, delta.parts, delta.weight, delta.eps, None, out)
+        K.postnorm_add_rmsnorm(h, delta.y, delta.parts, delta.weight, delta.eps, None, out, bias=delta.bias)
         return out
 
     def forward(self, h, delta, mixer, feed_forward, ctx, mem):
         from ..ops import kernels as K
 
         a = mixer.forward(self._stream(h, delta), ctx, mem)
-        pending = K.PendingNorm(*K.split_sublayer_output(a), self.norms[0].weight, self.norms[0].eps)
+        pending = K.pending_norm(a, self.norms[0].weight, self.norms[0].eps)
         if not self.has_feed_forward:
             return pending
         f = feed_forward.forward(self._stream(h, pending), ctx)
-        return K.PendingNorm(*K.split_sublayer_output(f), self.norms[1].weight, self.norms[1].eps)
+        return K.pending_norm(f, self.norms[1].weight, self.norms[1].eps)
 
 
 register_part("block", "prenorm", PreNormBlock)

@@ -75,9 +75,8 @@ class DenseMLP:
         z = K.linear(x, self.w_up)
         K.bias_act(z, self.b_up, self.activation)
         y = K.linear(z, self.w_down, partial_ok=True)       # the next norm adds the partial products
-        if self.b_down is not None:
-            K.add_bias(y, self.b_down)
-        return y
+        # the second bias is left to whoever takes the output: a block that norms it adds the bias in that kernel
+        return K.BiasedOutput(y, self.b_down) if self.b_down is not None else y
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

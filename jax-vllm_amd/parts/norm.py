@@ -51,7 +51,8 @@ class RMSNorm:
             # a sublayer's output that is normed on its own before it joins the stream: both norms in one pass
             n_out = h.shape[0] if rows is None else rows.numel()
             out = torch.empty((n_out, self.size), dtype=self.dtype, device=h.device)
-            K.postnorm_add_rmsnorm(h, delta.y, delta.parts, delta.weight, delta.eps, self.weight, out, rows, out_eps=self.eps)
+            K.postnorm_add_rmsnorm(h, delta.y, delta.parts, delta.weight, delta.eps, self.weight, out, rows, out_eps=self.eps,
+                                   bias=delta.bias)
             return out
         if (unscaled_ok and rows is None and delta is not None and delta.dim() == 3
                 and K.unscaled_rows_possible(self.dtype, h.shape[0], self.size)):

@@ -73,9 +73,8 @@ class Retention:
         H, d, dv = self.heads, self.dim, self.vdim
         proj = K.linear(x, self.w_in)
         cos_sin = self.position.rotation_table(ctx) if self.rot_dims else None
-        q = K.heads_to_f32(proj, 0, H, d, self.rot_dims, cos_sin)
-        k = K.heads_to_f32(proj, H * d, H, d, self.rot_dims, cos_sin, scale=d ** -0.5)
-        v = K.heads_to_f32(proj, 2 * H * d, H, dv)
+        qkv = K.qkv_to_f32(proj, H, d, dv, self.rot_dims, cos_sin, k_scale=d ** -0.5)
+        q, k, v = qkv[:, :H * d], qkv[:, H * d:2 * H * d], qkv[:, 2 * H * d:]
         o = K.recurrence_steps(q, k, v, self.decay, mem.states["S"], ctx.slot_ids, ctx.cu_seqlens, H, H, d, dv,
                                chunk_plan=K.step_chunk_plan(ctx, d))
         y = K.group_gated_norm(o, proj[:, 2 * H * d + H * dv:], None, dv, self.eps, "silu", out_scale=self.out_scale)

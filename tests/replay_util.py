@@ -108,7 +108,8 @@ def run_trace(model_dir, dtype, trace, max_tokens, out_dir, block_size=None, tim
     finally:
         if proc.poll() is None:
             proc.kill()
-    vocab = json.loads((Path(model_dir) / "config.json").read_text())["vocab_size"]
+    cfg = json.loads((Path(model_dir) / "config.json").read_text())
+    vocab = cfg["vocab_size"] if "vocab_size" in cfg else cfg["vocab"]
     out = {}
     for idx, rows in trace.rows.items():
         a = np.fromfile(Path(out_dir) / f"{idx}.f32", dtype="<f4")

@@ -307,6 +307,52 @@ def test_command_line_runs_the_design(folders, capsys):
     assert len(got) == 5
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_replay_with_four_slots_and_a_pool_for_the_live_requests_only(folders, dtype, tmp_path):
+    """``bin/trace_run`` on a mixed schedule: nine requests of 20 to 150 tokens, at most four live, portions of some
+    beside single tokens of others, some sitting a step out; the pool holds what the live requests hold at the peak, so
+    pages and slots are used again; then one request whole, one with its tail decoded, one in portions down to two."""
+    from tests.replay_util import Trace, compare, mixed, portions, run_trace, tail_one_by_one, whole
+
+    cfg, w = plain_of(folders["A"])
+    rng = np.random.default_rng(17)
+    reqs = {f"q{i}": tokens_of(cfg, n, 50 + i) for i, n in enumerate((150, 20, 77, 64, 33, 129, 48, 90, 65))}
+    trace = Trace()
+    peak = mixed(trace, reqs, rng)
+    whole(trace, "q0#w", reqs["q0"])
+    tail_one_by_one(trace, "q2#t", reqs["q2"], tail=40)
+    portions(trace, "q5#p", reqs["q5"], (2, 31, 3, 17))
+    got = run_trace(folders["A"], dtype, trace, max(peak, 192), tmp_path / "out", block_size=SMALL_A["page_size"])
+    want = {r: expected(cfg, w, t, dtype) for r, t in reqs.items()}
+    rows_got, rows_plain, rows_rounded = [], [], []
+
+    def collect(name, pos, got_row, want_row):
+        rows_got.append(got_row)
+        if dtype == "float32":
+            rows_plain.append(want_row)
+        else:
+            rows_plain.append(want_row[0][pos])
+            rows_rounded.append(want_row[1][pos])
+
+    if dtype == "float32":
+        n = compare(trace, got, want, collect)
+        check_rows(dtype, np.stack(rows_got), np.stack(rows_plain), "trace")
+    else:
+        n = compare(trace, got, {r: _Both(v) for r, v in want.items()}, collect)
+        check_rows(dtype, np.stack(rows_got), (np.stack(rows_plain), np.stack(rows_rounded)), "trace")
+    assert n == sum(len(t) for t in reqs.values()) + 150 + 41 + 129
+
+
+class _Both:
+    """(plain logits, plain logits with rounded products) of a request, indexed by position as one."""
+
+    def __init__(self, pair):
+        self.pair = pair
+
+    def __getitem__(self, pos):
+        return self.pair
+
+
 # ------------------------------------------------------------------ sizes that are no multiples of anything
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_odd_sizes_and_heads_beyond_the_matrix_core_kernels(tmp_path, dtype):
@@ -452,6 +498,11 @@ def test_gates_heads_and_norms_around_the_recurrence(dtype):
     got = K.heads_to_f32(proj.cuda(), 7, heads, d, 6, table, scale=0.3).cpu().double().view(n, heads, d)
     want = P.rotate(raw[:, 7:7 + heads * d].view(n, heads, d).transpose(0, 1), pos, r).transpose(0, 1) * 0.3
     assert float((got - want).abs().max()) < 1e-4 * float(want.abs().max())
+    both = K.qkv_to_f32(proj.cuda(), heads, d, 4, 6, table, k_scale=0.3).cpu().double()      # q, k and v of one mixer in one launch
+    wq = P.rotate(raw[:, :heads * d].view(n, heads, d).transpose(0, 1), pos, r).transpose(0, 1).reshape(n, -1)
+    wk = P.rotate(raw[:, heads * d:2 * heads * d].view(n, heads, d).transpose(0, 1), pos, r).transpose(0, 1).reshape(n, -1) * 0.3
+    wantb = torch.cat([wq, wk, raw[:, 2 * heads * d:2 * heads * d + heads * 4]], dim=1)
+    assert both.shape == wantb.shape and float((both - wantb).abs().max()) < 1e-4 * float(wantb.abs().max())
     x = torch.randn(n, 5 * d + 3, generator=gen)
     y = x.cuda().clone()
     K.head_unit_norm(y, 4, d, 1e-6, scale=2.0, first_heads=1, first_scale=0.5)
@@ -544,6 +595,13 @@ def test_bias_with_activation_stream_in_the_activation_type_and_weighed_sums(dty
     K.postnorm_add_rmsnorm(h, yy.cuda(), None, wb.cuda(), 1e-3, None, out)
     assert float((h.cpu().double() - want_h).abs().max()) <= 1e-5
     assert float((out.cpu().double() - want_h).abs().max()) <= tol * float(want_h.abs().max())
+    # a bias that the sublayer's output still owes is added before its norm, in rows of any width
+    for width in (52, 50):
+        bb = torch.randn(width, generator=gen)
+        want_b = h0[:, :width].double() + P.rms(yy[:, :width].double() + bb.double(), 1e-3) * wb[:width].double()
+        h = h0[:, :width].contiguous().cuda()
+        K.postnorm_add_rmsnorm(h, yy[:, :width].contiguous().cuda(), None, wb[:width].contiguous().cuda(), 1e-3, None, None, bias=bb.cuda())
+        assert float((h.cpu().double() - want_b).abs().max()) <= 1e-5, width
     parts = torch.randn(3, 9, 52, generator=gen)
     acc = torch.empty(9, 52, dtype=torch.float32, device="cuda")
     K.scaled_sum(acc, (yy.cuda(), parts.cuda()), 0.6)
