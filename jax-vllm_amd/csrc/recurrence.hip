@@ -402,7 +402,10 @@ recurrence_scan_kernel(float* __restrict__ scratch, float* __restrict__ state, c
   *S = s;
 }
 
-// grid as the local kernel
+// grid as the local kernel.  out[32 x LV] += diag(cum) Q[32 x dim] P[dim x LV] on the matrix cores in true 32-bit
+// (v_mfma_f32_32x32x2_f32: float operands, float products and sums): a wave takes 32 of the block's columns, its B
+// operands come straight from the state in global memory (every element is used by one wave only), A from LDS.
+typedef float rc_f32x16 __attribute__((ext_vector_type(16)));
 __global__ void __launch_bounds__(256)
 recurrence_apply_kernel(float* __restrict__ out, const float* __restrict__ scratch, const float* __restrict__ cum,
                         const float* __restrict__ q, long long ldq, const int* __restrict__ work,
@@ -414,44 +417,35 @@ recurrence_apply_kernel(float* __restrict__ out, const float* __restrict__ scrat
   const int hk = h / (heads / qk_heads);
   const int dq = dim + 1;
   float* qs = lds;                       // [LC][dq]
-  float* ps = qs + RC_LC * dq;           // [32][LV]: a slab of 32 rows of the state
   const int tid = threadIdx.x;
-  const int ncols = min(RC_LV, vdim - c0);
   for (int i = tid; i < RC_LC * dim; i += 256) {
     const int j = i / dim, d = i - j * dim;
     qs[j * dq + d] = j < n ? q[(long long)(b0 + j) * ldq + hk * dim + d] : 0.f;
   }
-  const float* P = scratch + (((long long)ch * heads + h) * dim) * vdim + c0;
-  const int i0 = (tid >> 5) * 4, c = (tid & 31) * 4;       // thread: rows i0..i0+3, columns c..c+3
-  float o[4][4] = {};
-  for (int d0 = 0; d0 < dim; d0 += 32) {
-    __syncthreads();
-    for (int e = tid; e < 32 * RC_LV; e += 256) {
-      const int d = d0 + e / RC_LV, cc = e % RC_LV;
-      ps[e] = (d < dim && cc < ncols) ? P[(long long)d * vdim + cc] : 0.f;
-    }
-    __syncthreads();
-    const int dn = min(32, dim - d0);
-    for (int d = 0; d < dn; ++d) {
-      const float4 p = *(const float4*)(ps + d * RC_LV + c);
-      const float pp[4] = {p.x, p.y, p.z, p.w};
-#pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        const float qv = qs[(i0 + a) * dq + d0 + d];
-#pragma unroll
-        for (int b = 0; b < 4; ++b) o[a][b] = fmaf(qv, pp[b], o[a][b]);
-      }
-    }
+  __syncthreads();
+  const int wave = tid / JV_WAVE, lane = tid % JV_WAVE;
+  const int wc0 = c0 + wave * 32;                          // this wave's first column
+  if (wc0 >= vdim) return;
+  const int col = lane % 32, kh = lane / 32;
+  const bool live = wc0 + col < vdim;
+  const float* P = scratch + (((long long)ch * heads + h) * dim) * vdim + wc0 + (live ? col : 0);
+  const float* A = qs + col * dq + kh;                     // row `col` of Q, elements kh, kh + 2, ...
+  rc_f32x16 acc = {};
+  // two products a turn (dim is a multiple of 4), their loads asked for together
+  for (int d = 0; d < dim; d += 4) {
+    const float b0v = P[(long long)(d + kh) * vdim], b1v = P[(long long)(d + 2 + kh) * vdim];
+    const float a0 = A[d], a1 = A[d + 2];
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, live ? b0v : 0.f, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, live ? b1v : 0.f, acc, 0, 0, 0);
   }
+  if (!live) return;
 #pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    const int i = i0 + a;
-    if (i >= n) continue;
-    const float w = cum ? cum[(long long)(b0 + i) * heads + h] : 1.f;
-    float* dst = out + (long long)(b0 + i) * heads * vdim + h * vdim + c0 + c;
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-      if (c + b < ncols) dst[b] += w * o[a][b];
+  for (int e = 0; e < 16; ++e) {
+    const int i = (e / 4) * 8 + kh * 4 + e % 4;            // the row of accumulator element e
+    if (i < n) {
+      const float w = cum ? cum[(long long)(b0 + i) * heads + h] : 1.f;
+      out[(long long)(b0 + i) * heads * vdim + h * vdim + wc0 + col] += w * acc[e];
+    }
   }
 }
 
@@ -472,7 +466,7 @@ extern "C" int jv_recurrence_chunks(float* out, const float* q, long long ldq, c
   hipStream_t s = (hipStream_t)stream;
   const int slices = (vdim + RC_LV - 1) / RC_LV;
   const size_t lds_local = (2 * RC_LC * (dim + RC_PAD) + RC_LC * RC_LV + RC_LC * (RC_LC + 1) + 2 * RC_LC) * sizeof(float);
-  const size_t lds_apply = (RC_LC * (dim + 1) + 32 * RC_LV) * sizeof(float);
+  const size_t lds_apply = (size_t)RC_LC * (dim + 1) * sizeof(float);
   hipLaunchKernelGGL(recurrence_local_kernel, dim3(chunks, heads, slices), dim3(256), lds_local, s, out, scratch, cum, q,
                      ldq, k, ldk, v, ldv, g, g_stride, wgt, skip, work, cu_seqlens, heads, qk_heads, dim, vdim);
   hipLaunchKernelGGL(recurrence_scan_kernel, dim3(n_requests, heads, (dim * vdim + 255) / 256), dim3(256), 0, s, scratch,
@@ -782,7 +776,7 @@ extern "C" int jv_delta_chunks(float* out, const float* q, long long ldq, const 
   float* qt = sb + per * dim * vdim;
   const size_t lds_local = (2 * RC_LC * (dim + RC_PAD) + 3 * RC_LC * (RC_LC + 1) + RC_LC * RC_LV + 3 * RC_LC) * sizeof(float);
   const size_t lds_scan = ((size_t)dim * RC_DS + 2 * RC_LC * (dim + RC_PAD) + RC_LC * (RC_DS + 4)) * sizeof(float);
-  const size_t lds_apply = (RC_LC * (dim + 1) + 32 * RC_LV) * sizeof(float);
+  const size_t lds_apply = (size_t)RC_LC * (dim + 1) * sizeof(float);
   hipLaunchKernelGGL(delta_local_kernel, dim3(chunks, heads), dim3(256), lds_local, s, out, wk, kd, wv, qt, cum, q, ldq,
                      k, ldk, v, ldv, g, g_stride, wgt, work, cu_seqlens, heads, qk_heads, dim, vdim);
   hipLaunchKernelGGL(delta_scan_kernel, dim3(n_requests, heads, (vdim + RC_DS - 1) / RC_DS), dim3(256), lds_scan, s, sb,
