@@ -256,7 +256,11 @@ recurrence_steps_kernel(float* __restrict__ out, const float* __restrict__ q, lo
 #define RC_LV 128       // columns (elements of v) a block takes
 #define RC_PAD 4        // row padding of q and k in LDS: rows stay 16-byte aligned
 
-// grid (chunks, heads, column slices of RC_LV); work: chunk -> (request, first token)
+// grid (chunks, heads, column slices of RC_LV); work: chunk -> (request, first token).  The three products run on the
+// matrix cores in true 32-bit (v_mfma_f32_32x32x2_f32): the scores q_i . k_j with the key size shared out to the four
+// waves, then per wave 32 of the block's columns: out = a V and U = K'^T V from the same operands of V, which come
+// straight from global memory (every element is used by one wave only).
+typedef float rc_f32x16 __attribute__((ext_vector_type(16)));
 __global__ void __launch_bounds__(256)
 recurrence_local_kernel(float* __restrict__ out, float* __restrict__ scratch, float* __restrict__ cum,
                         const float* __restrict__ q, long long ldq, const float* __restrict__ k, long long ldk,
@@ -268,15 +272,15 @@ recurrence_local_kernel(float* __restrict__ out, float* __restrict__ scratch, fl
   const int r = work[2 * ch], b0 = work[2 * ch + 1];
   const int n = min(RC_LC, cu_seqlens[r + 1] - b0);
   const int hk = h / (heads / qk_heads);
-  const int dq = dim + RC_PAD;
+  const int dq = dim + 1, lm = RC_LC + 1;
   float* qs = lds;                       // [LC][dq]
   float* ks = qs + RC_LC * dq;           // [LC][dq]
-  float* vs = ks + RC_LC * dq;           // [LC][LV]
-  float* as = vs + RC_LC * RC_LV;        // [LC][LC + 1]
-  float* cl = as + RC_LC * (RC_LC + 1);  // [LC] cumulative log decay
+  float* ps = ks + RC_LC * dq;           // [4][LC][LC + 1]: the waves' shares of the scores
+  float* as = ps + 4 * RC_LC * lm;       // [LC][LC + 1]
+  float* cl = as + RC_LC * lm;           // [LC] cumulative log decay
   float* ws = cl + RC_LC;                // [LC] write strengths
   const int tid = threadIdx.x;
-  const int ncols = min(RC_LV, vdim - c0);
+  const int wave = tid / JV_WAVE, lane = tid % JV_WAVE, col = lane % 32, kh = lane / 32;
   if (tid < RC_LC) {
     float lg = 0.f, w = 0.f;
     if (tid < n) {
@@ -293,86 +297,78 @@ recurrence_local_kernel(float* __restrict__ out, float* __restrict__ scratch, fl
     ws[tid] = w;
     if (blockIdx.z == 0 && tid < n) cum[(long long)(b0 + tid) * heads + h] = expf(lg);
   }
-  for (int i = tid; i < RC_LC * dq; i += 256) {
-    const int j = i / dq, d = i - j * dq;
+  for (int i = tid; i < RC_LC * dim; i += 256) {
+    const int j = i / dim, d = i - j * dim;
     float qv = 0.f, kv = 0.f;
-    if (j < n && d < dim) {
+    if (j < n) {
       qv = q[(long long)(b0 + j) * ldq + hk * dim + d];
       kv = k[(long long)(b0 + j) * ldk + hk * dim + d];
     }
-    qs[i] = qv;
-    ks[i] = kv;
-  }
-  for (int i = tid; i < RC_LC * RC_LV; i += 256) {
-    const int j = i / RC_LV, c = i % RC_LV;
-    vs[i] = (j < n && c < ncols) ? v[(long long)(b0 + j) * ldv + h * vdim + c0 + c] : 0.f;
+    qs[j * dq + d] = qv;
+    ks[j * dq + d] = kv;
   }
   __syncthreads();
-  // a: thread (i, 4 consecutive j)
-  {
-    const int i = tid >> 3, j0 = (tid & 7) * 4;
-    float dot[4] = {0.f, 0.f, 0.f, 0.f};
-    if (j0 <= i) {
-      for (int d = 0; d < dim; ++d) {
-        const float qv = qs[i * dq + d];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) dot[u] = fmaf(qv, ks[(j0 + u) * dq + d], dot[u]);
-      }
+  {  // scores: wave w sums over its quarter of the key elements, two a product (one a half wave)
+    const int share = dim / 4, d0 = wave * share;          // dim is a multiple of 4; a share may be odd
+    rc_f32x16 acc = {};
+    for (int d = 0; d < share; d += 2) {
+      const int dd = d0 + d + kh;
+      const bool in = d + kh < share;
+      const float a = in ? qs[col * dq + dd] : 0.f, bq = in ? ks[col * dq + dd] : 0.f;
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bq, acc, 0, 0, 0);
     }
+    float* mine = ps + wave * RC_LC * lm;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) mine[((e / 4) * 8 + kh * 4 + e % 4) * lm + col] = acc[e];
+  }
+  __syncthreads();
+  {  // a[i][j] = (q_i . k_j) exp(c_i - c_j) w_j (+ skip on the diagonal): thread (i, 4 consecutive j)
+    const int i = tid >> 3, j0 = (tid & 7) * 4;
     const float sk = skip ? skip[h] : 0.f;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = j0 + u;
       float a = 0.f;
-      if (j <= i && i < n) a = dot[u] * expf(cl[i] - cl[j]) * ws[j] + (j == i ? sk : 0.f);
-      as[i * (RC_LC + 1) + j] = a;
-    }
-  }
-  __syncthreads();
-  // k_j <- exp(c_(n-1) - c_j) w_j k_j (rows beyond the chunk are zero already); out = a v
-  for (int i = tid; i < RC_LC * dq; i += 256) {
-    const int j = i / dq;
-    if (j < n) ks[i] *= expf(cl[n - 1] - cl[j]) * ws[j];
-  }
-  for (int e = tid; e < RC_LC * (RC_LV / 4); e += 256) {
-    const int i = e / (RC_LV / 4), c = (e % (RC_LV / 4)) * 4;
-    if (i < n && c < ncols) {
-      float4 o = {0.f, 0.f, 0.f, 0.f};
-      for (int j = 0; j <= i; ++j) {
-        const float a = as[i * (RC_LC + 1) + j];
-        const float4 x = *(const float4*)(vs + j * RC_LV + c);
-        o.x = fmaf(a, x.x, o.x); o.y = fmaf(a, x.y, o.y); o.z = fmaf(a, x.z, o.z); o.w = fmaf(a, x.w, o.w);
+      if (j <= i && i < n) {
+        const float dot = (ps[i * lm + j] + ps[(RC_LC + i) * lm + j]) + (ps[(2 * RC_LC + i) * lm + j] + ps[(3 * RC_LC + i) * lm + j]);
+        a = dot * expf(cl[i] - cl[j]) * ws[j] + (j == i ? sk : 0.f);
       }
-      float* dst = out + (long long)(b0 + i) * heads * vdim + h * vdim + c0 + c;
-      dst[0] = o.x;
-      if (c + 1 < ncols) dst[1] = o.y;
-      if (c + 2 < ncols) dst[2] = o.z;
-      if (c + 3 < ncols) dst[3] = o.w;
+      as[i * lm + j] = a;
     }
   }
+  // k_j <- exp(c_(n-1) - c_j) w_j k_j (rows beyond the chunk are zero already)
+  for (int i = tid; i < RC_LC * dim; i += 256) {
+    const int j = i / dim, d = i - j * dim;
+    if (j < n) ks[j * dq + d] *= expf(cl[n - 1] - cl[j]) * ws[j];
+  }
   __syncthreads();
-  // U[d][c]: tiles of 4 x 4 per thread
-  float* U = scratch + (((long long)ch * heads + h) * dim) * vdim + c0;
-  const int dt = (dim + 3) / 4;
-  for (int e = tid; e < dt * (RC_LV / 4); e += 256) {
-    const int d0 = (e / (RC_LV / 4)) * 4, c = (e % (RC_LV / 4)) * 4;
-    if (c >= ncols) continue;
-    float u[4][4] = {};
-    for (int j = 0; j < n; ++j) {
-      const float4 kv = *(const float4*)(ks + j * dq + d0);
-      const float4 x = *(const float4*)(vs + j * RC_LV + c);
-      const float kk[4] = {kv.x, kv.y, kv.z, kv.w}, vv[4] = {x.x, x.y, x.z, x.w};
+  const int wc0 = c0 + wave * 32;                          // this wave's first column
+  if (wc0 >= vdim) return;
+  const bool live = wc0 + col < vdim;
+  const float* V = v + (long long)b0 * ldv + h * vdim + wc0 + (live ? col : 0);
+  const int tiles = (dim + 31) / 32;                       // row tiles of U, at most 4
+  rc_f32x16 o = {}, u0 = {}, u1 = {}, u2 = {}, u3 = {};
+  for (int j = 0; j < RC_LC; j += 2) {
+    const int jj = j + kh;
+    const float vv = V[(long long)min(jj, n - 1) * ldv];
+    const float bv = (live && jj < n) ? vv : 0.f;
+    o = __builtin_amdgcn_mfma_f32_32x32x2f32(as[col * lm + jj], bv, o, 0, 0, 0);
+    const float* kr = ks + jj * dq + col;                  // K'^T: row d = 32 t + col, column jj
+    u0 = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[0], bv, u0, 0, 0, 0);
+    if (tiles > 1) u1 = __builtin_amdgcn_mfma_f32_32x32x2f32(col + 32 < dim ? kr[32] : 0.f, bv, u1, 0, 0, 0);
+    if (tiles > 2) u2 = __builtin_amdgcn_mfma_f32_32x32x2f32(col + 64 < dim ? kr[64] : 0.f, bv, u2, 0, 0, 0);
+    if (tiles > 3) u3 = __builtin_amdgcn_mfma_f32_32x32x2f32(col + 96 < dim ? kr[96] : 0.f, bv, u3, 0, 0, 0);
+  }
+  if (!live) return;
+  float* U = scratch + (((long long)ch * heads + h) * dim) * vdim + wc0 + col;
 #pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) u[a][b] = fmaf(kk[a], vv[b], u[a][b]);
-    }
-#pragma unroll
-    for (int a = 0; a < 4; ++a)
-      if (d0 + a < dim)
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-          if (c + b < ncols) U[(long long)(d0 + a) * vdim + c + b] = u[a][b];
+  for (int e = 0; e < 16; ++e) {
+    const int i = (e / 4) * 8 + kh * 4 + e % 4;            // the row of accumulator element e
+    if (i < n) out[(long long)(b0 + i) * heads * vdim + h * vdim + wc0 + col] = o[e];
+    if (i < dim) U[(long long)i * vdim] = u0[e];
+    if (i + 32 < dim) U[(long long)(i + 32) * vdim] = u1[e];
+    if (i + 64 < dim) U[(long long)(i + 64) * vdim] = u2[e];
+    if (i + 96 < dim) U[(long long)(i + 96) * vdim] = u3[e];
   }
 }
 
@@ -405,7 +401,6 @@ recurrence_scan_kernel(float* __restrict__ scratch, float* __restrict__ state, c
 // grid as the local kernel.  out[32 x LV] += diag(cum) Q[32 x dim] P[dim x LV] on the matrix cores in true 32-bit
 // (v_mfma_f32_32x32x2_f32: float operands, float products and sums): a wave takes 32 of the block's columns, its B
 // operands come straight from the state in global memory (every element is used by one wave only), A from LDS.
-typedef float rc_f32x16 __attribute__((ext_vector_type(16)));
 __global__ void __launch_bounds__(256)
 recurrence_apply_kernel(float* __restrict__ out, const float* __restrict__ scratch, const float* __restrict__ cum,
                         const float* __restrict__ q, long long ldq, const int* __restrict__ work,
@@ -465,7 +460,7 @@ extern "C" int jv_recurrence_chunks(float* out, const float* q, long long ldq, c
     return (int)hipErrorInvalidValue;
   hipStream_t s = (hipStream_t)stream;
   const int slices = (vdim + RC_LV - 1) / RC_LV;
-  const size_t lds_local = (2 * RC_LC * (dim + RC_PAD) + RC_LC * RC_LV + RC_LC * (RC_LC + 1) + 2 * RC_LC) * sizeof(float);
+  const size_t lds_local = (2 * RC_LC * (dim + 1) + 5 * RC_LC * (RC_LC + 1) + 2 * RC_LC) * sizeof(float);
   const size_t lds_apply = (size_t)RC_LC * (dim + 1) * sizeof(float);
   hipLaunchKernelGGL(recurrence_local_kernel, dim3(chunks, heads, slices), dim3(256), lds_local, s, out, scratch, cum, q,
                      ldq, k, ldk, v, ldv, g, g_stride, wgt, skip, work, cu_seqlens, heads, qk_heads, dim, vdim);
