@@ -11,7 +11,7 @@
 #include "common.h"
 
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 attn_prepare_wide_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, long long ld,
                          const float* __restrict__ bias, const float* __restrict__ q_w,
                          const float* __restrict__ k_w, float eps, const float* __restrict__ cos_sin,
@@ -89,7 +89,9 @@ attn_prepare_wide_kernel(T* __restrict__ q_out, const T* __restrict__ qkv, long 
       return (int)hipErrorInvalidValue;                                                                         \
     const size_t shmem = (size_t)(nq + nkv) * dk * sizeof(float);                                               \
     if (shmem > 64 * 1024) return (int)hipErrorInvalidValue;                                                    \
-    hipLaunchKernelGGL(attn_prepare_wide_kernel<T>, dim3(n), dim3(256), shmem, (hipStream_t)stream, (T*)q_out,  \
+    /* few tokens of many wide heads (a decode step): more threads a token */                                  \
+    const int threads = (n <= 256 && (nq + nkv) * dp >= 4096) ? 1024 : 256;                                     \
+    hipLaunchKernelGGL(attn_prepare_wide_kernel<T>, dim3(n), dim3(threads), shmem, (hipStream_t)stream, (T*)q_out, \
                        (const T*)qkv, ld, bias, q_w, k_w, eps, cos_sin, rot_dims, slot_mapping, (T*)k_pages,    \
                        (T*)v_pages, page_size, nq, nkv, dk, dv, dp, v_scale);                                   \
     return JV_LAUNCH_CHECK();                                                                                   \

@@ -816,7 +816,7 @@ group_gated_norm_kernel(T* __restrict__ out, const float* __restrict__ o, const 
 
 // The same for wide groups: one block a (row, group).
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 group_gated_norm_block_kernel(T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ gate,
                               long long g_stride, const float* __restrict__ w, int w_period, int width, int group,
                               float eps, int gate_act, int gate_first, float out_scale) {
@@ -926,7 +926,9 @@ extern "C" int jv_recurrence_steps(float* out, const float* q, long long ldq, co
     const int groups = width / group;                                                                          \
     if (groups > 65535) return (int)hipErrorInvalidValue;                                                      \
     if (group >= 256) {                                                                                        \
-      hipLaunchKernelGGL(group_gated_norm_block_kernel<T>, dim3(n, groups), dim3(256), 0, (hipStream_t)stream, \
+      /* few rows of very wide groups (a decode step): more threads a row, the row's time is its chain of loads */ \
+      const int threads = (group >= 2048 && (long long)n * groups <= 256) ? 1024 : 256;                       \
+      hipLaunchKernelGGL(group_gated_norm_block_kernel<T>, dim3(n, groups), dim3(threads), 0, (hipStream_t)stream, \
                          (T*)out, o, (const T*)gate, g_stride, w, w_period, width, group, eps, gate_act,       \
                          gate_first, out_scale);                                                               \
       return JV_LAUNCH_CHECK();                                                                                \
