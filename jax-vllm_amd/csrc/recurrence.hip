@@ -633,7 +633,9 @@ delta_local_kernel(float* __restrict__ out, float* __restrict__ wk_out, float* _
 // A barrier that waits for the block's LDS traffic only: loads from global memory that were asked for a turn ahead stay
 // in flight across it (`__syncthreads` would wait for them too).
 __device__ __forceinline__ void rc_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-// grid (requests, heads, column slices of RC_DS)
+// grid (requests, heads, column slices of RC_DS).  Both products of a chunk run on the matrix cores in true 32-bit:
+// U = Wv - Wk S with the key size shared out to the four waves (their shares are added through LDS), then
+// S <- G S + Kd^T U with wave w owning rows 32 w .. 32 w + 31 of the slice in its accumulators for the whole walk.
 __global__ void __launch_bounds__(256)
 delta_scan_kernel(float* __restrict__ sb, float* __restrict__ state, const float* __restrict__ wk_in,
                   const float* __restrict__ kd_in, const float* __restrict__ wv_in, const float* __restrict__ cum,
@@ -643,17 +645,25 @@ delta_scan_kernel(float* __restrict__ sb, float* __restrict__ state, const float
   const int r = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * RC_DS;
   const int first = req_chunks[r], last = req_chunks[r + 1];
   if (last <= first) return;
-  const int dq = dim + RC_PAD, lu = RC_DS + 4;
-  float* ss = lds;                       // [dim][RC_DS]
-  float* wk = ss + dim * RC_DS;          // [LC][dq]
-  float* kd = wk + RC_LC * dq;           // [LC][dq]
-  float* us = kd + RC_LC * dq;           // [LC][RC_DS + 4]: Wv, then U
+  const int dq = dim + 1, lu = RC_DS + 1;
+  float* ss = lds;                       // [dim][RC_DS]: the slice of S, as the first product's operand
+  float* wkd = ss + dim * RC_DS;         // [LC][dq]: Wk, then Kd
+  float* us = wkd + RC_LC * dq;          // [LC][RC_DS + 1]: Wv, then U
+  float* ps = us + RC_LC * lu;           // [4][LC][RC_DS + 1]: the waves' shares of Wk S
   const int tid = threadIdx.x;
+  const int wave = tid / JV_WAVE, lane = tid % JV_WAVE, col = lane % 32, kh = lane / 32;
   const int ncols = min(RC_DS, vdim - c0);
+  const bool live = col < ncols;
   float* S = state + ((long long)slot_ids[r] * heads + h) * dim * vdim + c0;
   for (int e = tid; e < dim * RC_DS; e += 256) {
     const int d = e / RC_DS, c = e % RC_DS;
     ss[e] = c < ncols ? S[(long long)d * vdim + c] : 0.f;
+  }
+  rc_f32x16 acc;                         // rows 32 wave + (e / 4) * 8 + kh * 4 + e % 4 of column col
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int d = wave * 32 + (e / 4) * 8 + kh * 4 + e % 4;
+    acc[e] = (d < dim && live) ? S[(long long)d * vdim + col] : 0.f;
   }
   const int end = cu_seqlens[r + 1];
   // a chunk's Wk, Kd and Wv travel through registers: they are asked for a turn ahead, while the turn before computes
@@ -665,32 +675,31 @@ delta_scan_kernel(float* __restrict__ sb, float* __restrict__ state, const float
     const int e = tid + u * 256;
     at[u] = e < RC_LC * dim ? (e / dim) * dq + e % dim : -1;
   }
-  auto fetch = [&](int ch) {
+  auto fetch_w = [&](int ch) {
     const float* wk_c = wk_in + ((long long)ch * heads + h) * RC_LC * dim;
-    const float* kd_c = kd_in + ((long long)ch * heads + h) * RC_LC * dim;
     const float* wv_c = wv_in + ((long long)ch * heads + h) * RC_LC * vdim + c0;
 #pragma unroll
-    for (int u = 0; u < RK; ++u) {
-      const int e = min(tid + u * 256, RC_LC * dim - 1);       // a piece beyond the chunk reads its last element, unused
-      rw[u] = wk_c[e];
-      rk[u] = kd_c[e];
-    }
+    for (int u = 0; u < RK; ++u) rw[u] = wk_c[min(tid + u * 256, RC_LC * dim - 1)];   // beyond the chunk: its last element, unused
 #pragma unroll
     for (int u = 0; u < RU; ++u) {
       const int e = tid + u * 256, i = e / RC_DS, c = e % RC_DS;
       ru[u] = wv_c[(long long)i * vdim + min(c, ncols - 1)];
     }
   };
-  fetch(first);
+  auto fetch_k = [&](int ch) {
+    const float* kd_c = kd_in + ((long long)ch * heads + h) * RC_LC * dim;
+#pragma unroll
+    for (int u = 0; u < RK; ++u) rk[u] = kd_c[min(tid + u * 256, RC_LC * dim - 1)];
+  };
+  fetch_w(first);
+  fetch_k(first);
+  const int share = dim / 4, d0 = wave * share;            // dim is a multiple of 4; a share may be odd
   for (int ch = first; ch < last; ++ch) {
     float* sb_c = sb + ((long long)ch * heads + h) * dim * vdim + c0;
-    rc_lds_barrier();      // the turn before has read wk, kd, us and written ss
+    rc_lds_barrier();      // the turn before has written ss and read wkd and us
 #pragma unroll
     for (int u = 0; u < RK; ++u)
-      if (at[u] >= 0) {
-        wk[at[u]] = rw[u];
-        kd[at[u]] = rk[u];
-      }
+      if (at[u] >= 0) wkd[at[u]] = rw[u];
 #pragma unroll
     for (int u = 0; u < RU; ++u) {
       const int e = tid + u * 256, i = e / RC_DS, c = e % RC_DS;
@@ -701,49 +710,51 @@ delta_scan_kernel(float* __restrict__ sb, float* __restrict__ state, const float
       if (c < ncols) sb_c[(long long)d * vdim + c] = ss[e];
     }
     rc_lds_barrier();
-    fetch(min(ch + 1, last - 1));       // never conditional: the last turn asks for its own chunk again
-    {  // U = Wv - Wk S: thread (token i, 4 columns)
-      const int i = tid >> 3, c = (tid & 7) * 4;
-      float4 p = {0.f, 0.f, 0.f, 0.f};
-      for (int d = 0; d < dim; ++d) {
-        const float w = wk[i * dq + d];
-        const float4 x = *(const float4*)(ss + d * RC_DS + c);
-        p.x = fmaf(w, x.x, p.x); p.y = fmaf(w, x.y, p.y); p.z = fmaf(w, x.z, p.z); p.w = fmaf(w, x.w, p.w);
+    fetch_w(min(ch + 1, last - 1));     // never conditional: the last turn asks for its own chunk again
+    {  // this wave's share of Wk S
+      rc_f32x16 p = {};
+      for (int d = 0; d < share; d += 2) {
+        const int dd = d0 + d + kh;
+        const bool in = d + kh < share;
+        p = __builtin_amdgcn_mfma_f32_32x32x2f32(in ? wkd[col * dq + dd] : 0.f, in ? ss[dd * RC_DS + col] : 0.f, p, 0, 0, 0);
       }
-      float4* u = (float4*)(us + i * lu + c);
-      float4 w4 = *u;
-      w4.x -= p.x; w4.y -= p.y; w4.z -= p.z; w4.w -= p.w;
-      *u = w4;
+      float* mine = ps + wave * RC_LC * lu;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) mine[((e / 4) * 8 + kh * 4 + e % 4) * lu + col] = p[e];
     }
+    rc_lds_barrier();
+#pragma unroll
+    for (int u = 0; u < RK; ++u)
+      if (at[u] >= 0) wkd[at[u]] = rk[u];
+#pragma unroll
+    for (int u = 0; u < RU; ++u) {      // U = Wv - Wk S
+      const int e = tid + u * 256, o = (e / RC_DS) * lu + e % RC_DS;
+      us[o] -= (ps[o] + ps[RC_LC * lu + o]) + (ps[2 * RC_LC * lu + o] + ps[3 * RC_LC * lu + o]);
+    }
+    fetch_k(min(ch + 1, last - 1));
     rc_lds_barrier();
     const int b0 = work[2 * ch + 1];
     const int n = min(RC_LC, end - b0);
     const float gn = cum[(long long)(b0 + n - 1) * heads + h];
-    for (int e = tid; e < (dim / 4) * (RC_DS / 4); e += 256) {      // S = G S + Kd^T U: tiles of 4 x 4
-      const int d0 = (e / (RC_DS / 4)) * 4, c = (e % (RC_DS / 4)) * 4;
-      float acc[4][4];
+    if (wave * 32 < dim) {               // S = G S + Kd^T U: this wave's 32 rows
 #pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        const float4 x = *(const float4*)(ss + (d0 + a) * RC_DS + c);
-        acc[a][0] = gn * x.x; acc[a][1] = gn * x.y; acc[a][2] = gn * x.z; acc[a][3] = gn * x.w;
-      }
-      for (int j = 0; j < n; ++j) {
-        const float4 kv = *(const float4*)(kd + j * dq + d0);
-        const float4 uv = *(const float4*)(us + j * lu + c);
-        const float kk[4] = {kv.x, kv.y, kv.z, kv.w}, uu[4] = {uv.x, uv.y, uv.z, uv.w};
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-#pragma unroll
-          for (int b = 0; b < 4; ++b) acc[a][b] = fmaf(kk[a], uu[b], acc[a][b]);
+      for (int e = 0; e < 16; ++e) acc[e] *= gn;
+      const bool row_in = wave * 32 + col < dim;
+      for (int j = 0; j < RC_LC; j += 2) {
+        const int jj = j + kh;
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(row_in ? wkd[jj * dq + wave * 32 + col] : 0.f, us[jj * lu + col], acc, 0, 0, 0);
       }
 #pragma unroll
-      for (int a = 0; a < 4; ++a) *(float4*)(ss + (d0 + a) * RC_DS + c) = float4{acc[a][0], acc[a][1], acc[a][2], acc[a][3]};
+      for (int e = 0; e < 16; ++e) {
+        const int d = wave * 32 + (e / 4) * 8 + kh * 4 + e % 4;
+        if (d < dim) ss[d * RC_DS + col] = acc[e];
+      }
     }
   }
-  __syncthreads();
-  for (int e = tid; e < dim * RC_DS; e += 256) {
-    const int d = e / RC_DS, c = e % RC_DS;
-    if (c < ncols) S[(long long)d * vdim + c] = ss[e];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) {
+    const int d = wave * 32 + (e / 4) * 8 + kh * 4 + e % 4;
+    if (d < dim && live) S[(long long)d * vdim + col] = acc[e];
   }
 }
 
@@ -770,7 +781,7 @@ extern "C" int jv_delta_chunks(float* out, const float* q, long long ldq, const 
   float* sb = wv + per * RC_LC * vdim;
   float* qt = sb + per * dim * vdim;
   const size_t lds_local = (2 * RC_LC * (dim + RC_PAD) + 3 * RC_LC * (RC_LC + 1) + RC_LC * RC_LV + 3 * RC_LC) * sizeof(float);
-  const size_t lds_scan = ((size_t)dim * RC_DS + 2 * RC_LC * (dim + RC_PAD) + RC_LC * (RC_DS + 4)) * sizeof(float);
+  const size_t lds_scan = ((size_t)dim * RC_DS + RC_LC * (dim + 1) + 5 * RC_LC * (RC_DS + 1)) * sizeof(float);
   const size_t lds_apply = (size_t)RC_LC * (dim + 1) * sizeof(float);
   hipLaunchKernelGGL(delta_local_kernel, dim3(chunks, heads), dim3(256), lds_local, s, out, wk, kd, wv, qt, cum, q, ldq,
                      k, ldk, v, ldv, g, g_stride, wgt, work, cu_seqlens, heads, qk_heads, dim, vdim);
